@@ -1,0 +1,480 @@
+// C ABI of libmxgemm.so: argument validation and kernel dispatch.  See include/mxgemm.h.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "mx_common.h"
+
+namespace mx {
+
+static thread_local char g_err[512] = "";
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+namespace {
+
+inline bool is_elem(int d) { return d == MX_E4M3 || d == MX_E5M2 || d == MX_E2M1; }
+inline int64_t round256(int64_t b) { return (b + 255) & ~(int64_t)255; }
+
+const mx_gemm_opts kDefaultOpts = {sizeof(mx_gemm_opts), 0, MX_SCALE_2D, MX_SCALE_2D, MX_KERNEL_AUTO, 32, {0, 0}};
+
+int check_tensor(const mx_tensor* t, const char* name, int min_nd, int max_nd) {
+  if (!t) return set_error(MX_ERR_INVALID, "%s: null descriptor", name);
+  if (t->ndim < min_nd || t->ndim > max_nd)
+    return set_error(MX_ERR_SHAPE, "%s: expected %d..%d dimensions, got %d", name, min_nd, max_nd, t->ndim);
+  int64_t numel = 1;
+  for (int i = 0; i < t->ndim; ++i) {
+    if (t->shape[i] < 0) return set_error(MX_ERR_SHAPE, "%s: negative extent", name);
+    if (t->stride[i] < 0) return set_error(MX_ERR_LAYOUT, "%s: negative strides are not supported", name);
+    numel *= t->shape[i];
+  }
+  if (numel > 0 && !t->ptr) return set_error(MX_ERR_INVALID, "%s: null data pointer", name);
+  return MX_OK;
+}
+
+bool pair_supported_by_mfma(int a, int b) {
+  return (a == MX_E4M3 && b == MX_E4M3) || (a == MX_E5M2 && b == MX_E5M2) ||
+         (a == MX_E2M1 && b == MX_E2M1) || (a == MX_E4M3 && b == MX_E2M1);
+}
+
+// Checks the layout preconditions of the MFMA kernels for a K-contiguous operand with `rows` rows.
+// Returns nullptr if fine, otherwise the reason.
+const char* mfma_operand_issue(const void* ptr, int64_t rows, int64_t ld_bytes, int64_t k_stride,
+                               int fmt, int packed_ok) {
+  if (k_stride != 1) return "K axis is not contiguous";
+  if (fmt == MX_E2M1 && !packed_ok) return "FP4 operand is not packed along K";
+  if (((uintptr_t)ptr) % 16 != 0) return "base pointer is not 16-byte aligned";
+  if (ld_bytes % 16 != 0) return "row pitch is not a multiple of 16 bytes";
+  if (rows * ld_bytes >= ((int64_t)1 << 31)) return "operand spans 2 GiB or more";
+  return nullptr;
+}
+
+}  // namespace
+}  // namespace mx
+
+using namespace mx;
+
+extern "C" {
+
+int mx_version(void) { return MXGEMM_VERSION; }
+
+const char* mx_last_error(void) { return g_err; }
+
+int mx_device_check(void) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return set_error(MX_ERR_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return set_error(MX_ERR_DEVICE, "hipGetDeviceProperties: %s", hipGetErrorString(e));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return set_error(MX_ERR_DEVICE, "libmxgemm is built for gfx950 only, device is %s", prop.gcnArchName);
+  return MX_OK;
+}
+
+int64_t mx_packed_scale_bytes(int64_t rows, int64_t K) {
+  return round256(packed_scale_dwords(rows, K) * 4);
+}
+
+int64_t mx_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, const mx_gemm_opts* opts) {
+  const mx_gemm_opts& o = opts ? *opts : kDefaultOpts;
+  if (o.kernel == MX_KERNEL_GENERIC) return 0;
+  int64_t b = 0;
+  if (o.a_scale_layout != MX_SCALE_NATIVE) b += mx_packed_scale_bytes(M, K);
+  if (o.b_scale_layout != MX_SCALE_NATIVE) b += mx_packed_scale_bytes(N, K);
+  return b;
+}
+
+int64_t mx_gemm_grouped_workspace_bytes(int64_t num_slots, int64_t N, int64_t K, int64_t E,
+                                        const mx_gemm_opts* opts) {
+  const mx_gemm_opts& o = opts ? *opts : kDefaultOpts;
+  if (o.kernel == MX_KERNEL_GENERIC) return 0;
+  int64_t b = mx_packed_scale_bytes(num_slots, K);
+  if (o.b_scale_layout != MX_SCALE_NATIVE) b += E * mx_packed_scale_bytes(N, K);
+  return b;
+}
+
+int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, void* packed,
+                   void* stream) {
+  if (int rc = check_tensor(scale, "scale", 2, 4)) return rc;
+  if (!packed) return set_error(MX_ERR_INVALID, "packed: null pointer");
+  if (K % 32 != 0) return set_error(MX_ERR_SHAPE, "K (%lld) must be a multiple of 32", (long long)K);
+  if (((uintptr_t)packed) % 16 != 0) return set_error(MX_ERR_LAYOUT, "packed buffer must be 16-byte aligned");
+  PackArgs p = {};
+  p.src = (const uint8_t*)scale->ptr;
+  p.dst = (uint32_t*)packed;
+  p.rows = rows;
+  p.K = K;
+  p.layout = layout;
+  p.batch = 1;
+  p.replicas = 1;
+  const int64_t KB = K / 32;
+  if (layout == MX_SCALE_2D) {
+    const int nd = scale->ndim;
+    if (nd != 2 && nd != 3) return set_error(MX_ERR_SHAPE, "2-D scale layout expects [rows, K/32] with an optional batch");
+    if (scale->shape[nd - 2] != rows || scale->shape[nd - 1] != KB)
+      return set_error(MX_ERR_SHAPE, "scale shape (%lld, %lld) does not match rows=%lld, K/32=%lld",
+                       (long long)scale->shape[nd - 2], (long long)scale->shape[nd - 1], (long long)rows,
+                       (long long)KB);
+    p.s_row = scale->stride[nd - 2];
+    p.s_kb = scale->stride[nd - 1];
+    if (nd == 3) {
+      p.batch = (int32_t)scale->shape[0];
+      p.s_batch = scale->stride[0];
+    }
+  } else if (layout == MX_SCALE_SWIZZLE_32_4_4) {
+    if (scale->ndim != 4 || scale->shape[2] != 32 || scale->shape[3] != 16)
+      return set_error(MX_ERR_SHAPE, "swizzled scale layout expects [rows/128, K/128, 32, 16]");
+    if (rows % 128 != 0 || KB % 4 != 0 || scale->shape[0] != rows / 128 || scale->shape[1] != KB / 4)
+      return set_error(MX_ERR_SHAPE, "swizzled scale shape does not match rows=%lld, K=%lld", (long long)rows,
+                       (long long)K);
+    if (scale->stride[3] != 1 || scale->stride[2] != 16 || scale->stride[1] != 512 ||
+        scale->stride[0] != 512 * (KB / 4))
+      return set_error(MX_ERR_LAYOUT, "swizzled scale tensor must be contiguous");
+  } else {
+    return set_error(MX_ERR_INVALID, "mx_pack_scales: unknown source layout %d", layout);
+  }
+  return launch_pack_scales(p, (hipStream_t)stream);
+}
+
+int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const mx_tensor* Bs, mx_tensor* C,
+            const mx_gemm_opts* opts, void* workspace, int64_t workspace_bytes, void* stream) {
+  const mx_gemm_opts& o = opts ? *opts : kDefaultOpts;
+  if (int rc = check_tensor(A, "A", 2, 3)) return rc;
+  if (int rc = check_tensor(B, "B", 2, 3)) return rc;
+  if (int rc = check_tensor(As, "A_scale", 2, 4)) return rc;
+  if (int rc = check_tensor(Bs, "B_scale", 2, 4)) return rc;
+  if (int rc = check_tensor(C, "C", 2, 3)) return rc;
+  if (!is_elem(A->dtype) || !is_elem(B->dtype))
+    return set_error(MX_ERR_DTYPE, "A/B must be MX_E4M3, MX_E5M2 or MX_E2M1 (got %d, %d)", A->dtype, B->dtype);
+  if (C->dtype != MX_F32 && C->dtype != MX_BF16)
+    return set_error(MX_ERR_DTYPE, "C must be MX_F32 or MX_BF16 (got %d)", C->dtype);
+  if (As->dtype != Bs->dtype) return set_error(MX_ERR_DTYPE, "A_scale and B_scale must have the same dtype");
+  if (As->dtype != MX_E8M0 && As->dtype != MX_E4M3)
+    return set_error(MX_ERR_DTYPE, "scale dtype must be MX_E8M0 (or MX_E4M3 for FP4 with block 16)");
+  if (o.block_size != 32 && o.block_size != 16)
+    return set_error(MX_ERR_INVALID, "block_size must be 16 or 32 (got %d)", o.block_size);
+
+  const int and_ = A->ndim, bnd = B->ndim, cnd = C->ndim;
+  const int64_t M = A->shape[and_ - 2], K = A->shape[and_ - 1];
+  const int64_t Kb = B->shape[bnd - 2], N = B->shape[bnd - 1];
+  if (K != Kb)
+    return set_error(MX_ERR_SHAPE, "Incompatible matrices: K dimension of A (%lld) must match K dimension of B (%lld)",
+                     (long long)K, (long long)Kb);
+  if (K % o.block_size != 0)
+    return set_error(MX_ERR_SHAPE, "K (%lld) must be a multiple of the scaling block size %d", (long long)K,
+                     o.block_size);
+  const int64_t batchA = and_ == 3 ? A->shape[0] : 1, batchB = bnd == 3 ? B->shape[0] : 1;
+  if (batchA != batchB && batchA != 1 && batchB != 1)
+    return set_error(MX_ERR_SHAPE, "batch dimensions %lld and %lld cannot be broadcast", (long long)batchA,
+                     (long long)batchB);
+  const int64_t batch = batchA > batchB ? batchA : batchB;
+  const bool batched = and_ == 3 || bnd == 3;
+  if ((batched && (cnd != 3 || C->shape[0] != batch)) || (!batched && cnd != 2) || C->shape[cnd - 2] != M ||
+      C->shape[cnd - 1] != N)
+    return set_error(MX_ERR_SHAPE, "C has the wrong shape for a (%lld x %lld x %lld) product", (long long)M,
+                     (long long)N, (long long)K);
+  if (A->dtype == MX_E2M1 && A->packed_dim != and_ - 1 && A->packed_dim != and_ - 2)
+    return set_error(MX_ERR_LAYOUT, "A: packed_dim must name the M or K dimension");
+  if (B->dtype == MX_E2M1 && B->packed_dim != bnd - 1 && B->packed_dim != bnd - 2)
+    return set_error(MX_ERR_LAYOUT, "B: packed_dim must name the K or N dimension");
+  const int64_t KB = K / o.block_size;
+
+  // ---- scale shapes --------------------------------------------------------------------------------
+  if (o.a_scale_layout == MX_SCALE_2D) {
+    const int nd = As->ndim;
+    if (nd != and_ || As->shape[nd - 2] != M || As->shape[nd - 1] != KB || (nd == 3 && As->shape[0] != batchA))
+      return set_error(MX_ERR_SHAPE, "A_scale shape is not compatible with A: expected [.., %lld, %lld]",
+                       (long long)M, (long long)KB);
+  }
+  if (o.b_scale_layout == MX_SCALE_2D) {
+    const int nd = Bs->ndim;
+    if (nd != bnd || Bs->shape[nd - 2] != KB || Bs->shape[nd - 1] != N || (nd == 3 && Bs->shape[0] != batchB))
+      return set_error(MX_ERR_SHAPE, "B_scale shape is not compatible with B: expected [.., %lld, %lld]",
+                       (long long)KB, (long long)N);
+  }
+  if (M == 0 || N == 0) return MX_OK;
+
+  // ---- can the MFMA path take it? ------------------------------------------------------------------
+  const char* why = nullptr;
+  const int64_t a_ld = A->stride[and_ - 2], b_ld = B->stride[bnd - 1];
+  if (batched) why = "batched operands";
+  else if (o.block_size != 32 || As->dtype != MX_E8M0) why = "only E8M0 scales with block 32 are MFMA-native";
+  else if (!pair_supported_by_mfma(A->dtype, B->dtype)) why = "element format pair not instantiated";
+  else if (K == 0) why = "K is zero";
+  else if ((why = mfma_operand_issue(A->ptr, M, a_ld, A->stride[1], A->dtype, A->packed_dim == 1))) {}
+  else if ((why = mfma_operand_issue(B->ptr, N, b_ld, B->stride[0], B->dtype, B->packed_dim == 0))) {}
+  else if (C->stride[1] != 1) why = "C is not row-major";
+  else if (M >= (1 << 30) || N >= (1 << 30) || K >= (1 << 30)) why = "extent too large";
+
+  int kernel = o.kernel;
+  if (kernel == MX_KERNEL_AUTO) {
+    if (why) kernel = MX_KERNEL_GENERIC;
+    else if (M <= 32 && A->dtype != MX_E2M1 && B->dtype == MX_E2M1 && o.a_scale_layout == MX_SCALE_2D &&
+             o.b_scale_layout == MX_SCALE_2D && Bs->stride[0] == 1 && As->stride[1] == 1 && K % 512 == 0 &&
+             K <= 8192 && N % 16 == 0 && Bs->stride[1] % 16 == 0 && ((uintptr_t)Bs->ptr) % 16 == 0)
+      kernel = MX_KERNEL_DECODE;
+    else if (M > 128 && N > 128 && (int64_t)M * N >= (int64_t)1024 * 1024) kernel = MX_KERNEL_MFMA_256x256;
+    else kernel = MX_KERNEL_MFMA_128x128;
+  } else if (kernel != MX_KERNEL_GENERIC && why) {
+    return set_error(MX_ERR_LAYOUT, "requested kernel %d cannot run this problem: %s", kernel, why);
+  }
+
+  if (kernel == MX_KERNEL_GENERIC) {
+    if (o.a_scale_layout == MX_SCALE_NATIVE || o.b_scale_layout == MX_SCALE_NATIVE)
+      return set_error(MX_ERR_LAYOUT, "the generic kernel cannot read native-layout scales");
+    if (As->dtype == MX_E4M3 && !(A->dtype == MX_E2M1 && o.block_size == 16))
+      return set_error(MX_ERR_DTYPE, "E4M3 scales are only defined for FP4 operands with block size 16");
+    if (o.block_size == 16 && (A->dtype != MX_E2M1 || B->dtype != MX_E2M1))
+      return set_error(MX_ERR_DTYPE, "block size 16 is only defined for FP4 operands");
+    GenericArgs g = {};
+    g.A = (const uint8_t*)A->ptr; g.As = (const uint8_t*)As->ptr;
+    g.B = (const uint8_t*)B->ptr; g.Bs = (const uint8_t*)Bs->ptr; g.C = C->ptr;
+    g.batch = (int32_t)batch; g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)K; g.block = o.block_size;
+    g.a_fmt = A->dtype; g.b_fmt = B->dtype; g.scale_fmt = As->dtype; g.c_dtype = C->dtype;
+    g.accumulate = o.accumulate;
+    g.a_packed_k = A->packed_dim == and_ - 1; g.b_packed_k = B->packed_dim == bnd - 2;
+    g.a_sb = (and_ == 3 && batchA > 1) ? A->stride[0] : 0;
+    g.a_sm = A->stride[and_ - 2]; g.a_sk = A->stride[and_ - 1];
+    g.b_sb = (bnd == 3 && batchB > 1) ? B->stride[0] : 0;
+    g.b_sk = B->stride[bnd - 2]; g.b_sn = B->stride[bnd - 1];
+    g.as_layout = o.a_scale_layout; g.bs_layout = o.b_scale_layout;
+    if (o.a_scale_layout == MX_SCALE_2D) {
+      const int nd = As->ndim;
+      g.as_sb = (nd == 3 && batchA > 1) ? As->stride[0] : 0;
+      g.as_sm = As->stride[nd - 2]; g.as_sk = As->stride[nd - 1];
+    } else if (M % 128 != 0 || KB % 4 != 0) {
+      return set_error(MX_ERR_SHAPE, "swizzled A_scale needs M %% 128 == 0 and (K/32) %% 4 == 0");
+    }
+    if (o.b_scale_layout == MX_SCALE_2D) {
+      const int nd = Bs->ndim;
+      g.bs_sb = (nd == 3 && batchB > 1) ? Bs->stride[0] : 0;
+      g.bs_sk = Bs->stride[nd - 2]; g.bs_sn = Bs->stride[nd - 1];
+    } else if (N % 128 != 0 || KB % 4 != 0) {
+      return set_error(MX_ERR_SHAPE, "swizzled B_scale needs N %% 128 == 0 and (K/32) %% 4 == 0");
+    }
+    g.c_sb = cnd == 3 ? C->stride[0] : 0; g.c_sm = C->stride[cnd - 2]; g.c_sn = C->stride[cnd - 1];
+    return launch_gemm_generic(g, (hipStream_t)stream);
+  }
+
+  if (kernel == MX_KERNEL_DECODE) {
+    if (M > 32) return set_error(MX_ERR_SHAPE, "the decode kernel handles M <= 32 (got %lld)", (long long)M);
+    if (o.a_scale_layout != MX_SCALE_2D || o.b_scale_layout != MX_SCALE_2D || Bs->stride[0] != 1 ||
+        As->stride[1] != 1)
+      return set_error(MX_ERR_LAYOUT, "the decode kernel reads K-contiguous 2-D scales in place");
+    if (A->dtype == MX_E2M1 || B->dtype != MX_E2M1)
+      return set_error(MX_ERR_DTYPE, "the decode kernel takes 8-bit activations and FP4 weights");
+    if (K % 512 != 0 || N % 16 != 0)
+      return set_error(MX_ERR_SHAPE, "the decode kernel needs K %% 512 == 0 and N %% 16 == 0");
+    DecodeArgs d = {};
+    d.X = (const uint8_t*)A->ptr; d.Xs = (const uint8_t*)As->ptr;
+    d.W = (const uint8_t*)B->ptr; d.Ws = (const uint8_t*)Bs->ptr; d.C = C->ptr;
+    d.M = (int32_t)M; d.N = (int32_t)N; d.K = (int32_t)K;
+    d.ldx = a_ld; d.ldxs = As->stride[0]; d.ldw = b_ld; d.ldws = Bs->stride[1]; d.ldc = C->stride[0];
+    d.x_fmt = A->dtype; d.w_fmt = B->dtype; d.c_dtype = C->dtype; d.accumulate = o.accumulate;
+    return launch_gemm_decode(d, (hipStream_t)stream);
+  }
+
+  // ---- MFMA path: bring the scales into the native layout if they are not ----------------------------
+  uint8_t* ws = (uint8_t*)workspace;
+  int64_t need = mx_gemm_workspace_bytes(M, N, K, &o);
+  if (need > 0 && (!ws || workspace_bytes < need))
+    return set_error(MX_ERR_WORKSPACE, "workspace of %lld bytes required, %lld given", (long long)need,
+                     (long long)workspace_bytes);
+  if (need > 0 && ((uintptr_t)ws) % 256 != 0)
+    return set_error(MX_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  const uint32_t* as_native = (const uint32_t*)As->ptr;
+  const uint32_t* bs_native = (const uint32_t*)Bs->ptr;
+  if (o.a_scale_layout != MX_SCALE_NATIVE) {
+    if (int rc = mx_pack_scales(As, o.a_scale_layout, M, K, ws, stream)) return rc;
+    as_native = (const uint32_t*)ws;
+    ws += mx_packed_scale_bytes(M, K);
+  }
+  if (o.b_scale_layout != MX_SCALE_NATIVE) {
+    mx_tensor t = *Bs;
+    if (o.b_scale_layout == MX_SCALE_2D) {  // [K/32, N] -> view as [N, K/32]
+      t.shape[0] = Bs->shape[1]; t.shape[1] = Bs->shape[0];
+      t.stride[0] = Bs->stride[1]; t.stride[1] = Bs->stride[0];
+    }
+    if (int rc = mx_pack_scales(&t, o.b_scale_layout, N, K, ws, stream)) return rc;
+    bs_native = (const uint32_t*)ws;
+  }
+  if (((uintptr_t)as_native) % 16 != 0 || ((uintptr_t)bs_native) % 16 != 0)
+    return set_error(MX_ERR_LAYOUT, "native scale buffers must be 16-byte aligned");
+
+  GemmArgs g = {};
+  g.A = (const uint8_t*)A->ptr; g.B = (const uint8_t*)B->ptr; g.As = as_native; g.Bs = bs_native; g.C = C->ptr;
+  g.lda = a_ld; g.ldb = b_ld; g.ldc = C->stride[0];
+  g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)K;
+  g.a_fmt = A->dtype; g.b_fmt = B->dtype; g.c_dtype = C->dtype; g.accumulate = o.accumulate;
+  g.a_rows = M;
+  g.replicas = 1;
+  return launch_gemm_mfma(g, kernel, (hipStream_t)stream);
+}
+
+int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W, const mx_tensor* Ws,
+                    mx_tensor* C, const float* topk_weights, const int32_t* sorted_token_ids,
+                    int64_t num_slots, const int32_t* sorted_expert_ids, int32_t tile_m,
+                    int32_t num_token_replicas, int64_t num_valid_ids, const mx_gemm_opts* opts,
+                    void* workspace, int64_t workspace_bytes, void* stream) {
+  const mx_gemm_opts& o = opts ? *opts : kDefaultOpts;
+  if (int rc = check_tensor(A, "A", 2, 2)) return rc;
+  if (int rc = check_tensor(As, "A_scale", 2, 2)) return rc;
+  if (int rc = check_tensor(W, "W", 3, 3)) return rc;
+  if (int rc = check_tensor(Ws, "W_scale", 3, 3)) return rc;
+  if (int rc = check_tensor(C, "C", 2, 2)) return rc;
+  if (!sorted_token_ids || !sorted_expert_ids) return set_error(MX_ERR_INVALID, "null index arrays");
+  if (tile_m <= 0 || num_slots % tile_m != 0)
+    return set_error(MX_ERR_SHAPE, "num_slots (%lld) must be a multiple of tile_m (%d)", (long long)num_slots, tile_m);
+  if (num_token_replicas <= 0) return set_error(MX_ERR_INVALID, "num_token_replicas must be positive");
+  if (!is_elem(A->dtype) || !is_elem(W->dtype)) return set_error(MX_ERR_DTYPE, "A/W must be MX element formats");
+  if (As->dtype != MX_E8M0 || Ws->dtype != MX_E8M0) return set_error(MX_ERR_DTYPE, "scales must be MX_E8M0");
+  if (C->dtype != MX_F32 && C->dtype != MX_BF16) return set_error(MX_ERR_DTYPE, "C must be MX_F32 or MX_BF16");
+  if (o.block_size != 32) return set_error(MX_ERR_INVALID, "grouped GEMM supports block size 32 only");
+  const int64_t T = A->shape[0], K = A->shape[1], E = W->shape[0], N = W->shape[1];
+  if (W->shape[2] != K)
+    return set_error(MX_ERR_SHAPE, "Incompatible matrices: K dimension of A (%lld) must match K dimension of W (%lld)",
+                     (long long)K, (long long)W->shape[2]);
+  if (K % 32 != 0) return set_error(MX_ERR_SHAPE, "K (%lld) must be a multiple of 32", (long long)K);
+  const int64_t KB = K / 32;
+  if (As->shape[0] != T || As->shape[1] != KB) return set_error(MX_ERR_SHAPE, "A_scale must be [tokens, K/32]");
+  if (o.b_scale_layout != MX_SCALE_NATIVE && (Ws->shape[0] != E || Ws->shape[1] != N || Ws->shape[2] != KB))
+    return set_error(MX_ERR_SHAPE, "W_scale must be [experts, N, K/32]");
+  if (C->shape[1] != N || C->shape[0] < num_valid_ids)
+    return set_error(MX_ERR_SHAPE, "C must be [>= num_valid_ids, N]");
+  if ((num_valid_ids + num_token_replicas - 1) / num_token_replicas > T)
+    return set_error(MX_ERR_SHAPE, "num_valid_ids / num_token_replicas exceeds the rows of A");
+  if (num_slots == 0 || N == 0) return MX_OK;
+  if (A->dtype == MX_E2M1 && A->packed_dim != 1) return set_error(MX_ERR_LAYOUT, "A must be packed along K");
+  if (W->dtype == MX_E2M1 && W->packed_dim != 2) return set_error(MX_ERR_LAYOUT, "W must be packed along K");
+
+  const char* why = nullptr;
+  if (!pair_supported_by_mfma(A->dtype, W->dtype)) why = "element format pair not instantiated";
+  else if ((why = mfma_operand_issue(A->ptr, T, A->stride[0], A->stride[1], A->dtype, 1))) {}
+  else if ((why = mfma_operand_issue(W->ptr, N, W->stride[1], W->stride[2], W->dtype, 1))) {}
+  else if (W->stride[0] % 16 != 0) why = "expert pitch of W is not a multiple of 16 bytes";
+  else if (C->stride[1] != 1) why = "C is not row-major";
+  else if (tile_m % 128 != 0) why = "tile_m is not a multiple of 128";
+  else if (o.a_scale_layout != MX_SCALE_2D) why = "A_scale must be the plain 2-D layout";
+
+  int kernel = o.kernel;
+  if (kernel == MX_KERNEL_AUTO) {
+    if (why) kernel = MX_KERNEL_GENERIC;
+    else kernel = (tile_m % 256 == 0 && N > 128) ? MX_KERNEL_MFMA_256x256 : MX_KERNEL_MFMA_128x128;
+  } else if (kernel != MX_KERNEL_GENERIC) {
+    if (why) return set_error(MX_ERR_LAYOUT, "requested kernel %d cannot run this problem: %s", kernel, why);
+    const int bm = kernel == MX_KERNEL_MFMA_128x128 ? 128 : 256;
+    if (kernel == MX_KERNEL_DECODE || tile_m % bm != 0)
+      return set_error(MX_ERR_LAYOUT, "kernel %d needs tile_m to be a multiple of its row tile", kernel);
+  }
+
+  if (kernel == MX_KERNEL_GENERIC) {
+    if (o.a_scale_layout != MX_SCALE_2D || o.b_scale_layout != MX_SCALE_2D)
+      return set_error(MX_ERR_LAYOUT, "the generic grouped kernel reads plain 2-D / 3-D scales");
+    GenericArgs g = {};
+    g.A = (const uint8_t*)A->ptr; g.As = (const uint8_t*)As->ptr;
+    g.B = (const uint8_t*)W->ptr; g.Bs = (const uint8_t*)Ws->ptr; g.C = C->ptr;
+    g.batch = 1; g.M = (int32_t)T; g.N = (int32_t)N; g.K = (int32_t)K; g.block = 32;
+    g.a_fmt = A->dtype; g.b_fmt = W->dtype; g.scale_fmt = MX_E8M0; g.c_dtype = C->dtype; g.accumulate = o.accumulate;
+    g.a_packed_k = 1; g.b_packed_k = 1;
+    g.a_sm = A->stride[0]; g.a_sk = A->stride[1];
+    g.as_sm = As->stride[0]; g.as_sk = As->stride[1];
+    g.b_sn = W->stride[1]; g.b_sk = W->stride[2]; g.b_se = W->stride[0];
+    g.bs_sn = Ws->stride[1]; g.bs_sk = Ws->stride[2]; g.bs_se = Ws->stride[0];
+    g.c_sm = C->stride[0]; g.c_sn = C->stride[1];
+    g.sorted_token_ids = sorted_token_ids; g.sorted_expert_ids = sorted_expert_ids; g.topk_weights = topk_weights;
+    g.tile_m = tile_m; g.replicas = num_token_replicas; g.num_valid_ids = num_valid_ids; g.num_slots = num_slots;
+    return launch_gemm_generic(g, (hipStream_t)stream);
+  }
+
+  uint8_t* ws = (uint8_t*)workspace;
+  const int64_t need = mx_gemm_grouped_workspace_bytes(num_slots, N, K, E, &o);
+  if (!ws || workspace_bytes < need)
+    return set_error(MX_ERR_WORKSPACE, "workspace of %lld bytes required, %lld given", (long long)need,
+                     (long long)workspace_bytes);
+  if (((uintptr_t)ws) % 256 != 0) return set_error(MX_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  // A scales: gathered into slot order while re-laying
+  {
+    PackArgs p = {};
+    p.src = (const uint8_t*)As->ptr; p.dst = (uint32_t*)ws;
+    p.rows = num_slots; p.K = K; p.s_row = As->stride[0]; p.s_kb = As->stride[1];
+    p.layout = MX_SCALE_2D; p.batch = 1;
+    p.gather_ids = sorted_token_ids; p.replicas = num_token_replicas; p.num_valid_ids = num_valid_ids;
+    if (int rc = launch_pack_scales(p, (hipStream_t)stream)) return rc;
+  }
+  const uint32_t* as_native = (const uint32_t*)ws;
+  ws += mx_packed_scale_bytes(num_slots, K);
+  const uint32_t* bs_native = (const uint32_t*)Ws->ptr;
+  if (o.b_scale_layout != MX_SCALE_NATIVE) {
+    if (o.b_scale_layout != MX_SCALE_2D) return set_error(MX_ERR_LAYOUT, "W_scale must be [E, N, K/32] or native");
+    if (int rc = mx_pack_scales(Ws, MX_SCALE_2D, N, K, ws, stream)) return rc;
+    bs_native = (const uint32_t*)ws;
+  }
+  GemmArgs g = {};
+  g.A = (const uint8_t*)A->ptr; g.B = (const uint8_t*)W->ptr; g.As = as_native; g.Bs = bs_native; g.C = C->ptr;
+  g.lda = A->stride[0]; g.ldb = W->stride[1]; g.ldc = C->stride[0];
+  g.M = (int32_t)num_slots; g.N = (int32_t)N; g.K = (int32_t)K;
+  g.a_fmt = A->dtype; g.b_fmt = W->dtype; g.c_dtype = C->dtype; g.accumulate = o.accumulate;
+  g.sorted_token_ids = sorted_token_ids; g.sorted_expert_ids = sorted_expert_ids; g.topk_weights = topk_weights;
+  g.tile_m = tile_m; g.replicas = num_token_replicas; g.num_valid_ids = num_valid_ids;
+  g.b_expert_stride = W->stride[0];
+  g.bs_expert_stride = mx_packed_scale_bytes(N, K) / 4;
+  g.a_rows = T;
+  return launch_gemm_mfma(g, kernel, (hipStream_t)stream);
+}
+
+int64_t mx_moe_align_max_slots(int64_t num_ids, int32_t num_experts, int32_t tile_m) {
+  if (num_ids < 0 || num_experts <= 0 || tile_m <= 0) return 0;
+  const int64_t nonempty = num_experts < num_ids ? num_experts : num_ids;
+  return (num_ids + nonempty * (tile_m - 1)) / tile_m * tile_m;
+}
+
+int mx_moe_align(const int32_t* topk_ids, int64_t num_ids, int32_t num_experts, int32_t tile_m,
+                 int32_t* sorted_token_ids, int32_t* sorted_expert_ids, int32_t* num_slots_out, void* stream) {
+  if (num_ids < 0 || num_experts <= 0 || tile_m <= 0) return set_error(MX_ERR_INVALID, "moe_align: bad sizes");
+  if (num_ids >= 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "moe_align: too many ids");
+  const int64_t max_slots = mx_moe_align_max_slots(num_ids, num_experts, tile_m);
+  if (max_slots == 0) {
+    return MX_OK;
+  }
+  if (!topk_ids || !sorted_token_ids || !sorted_expert_ids) return set_error(MX_ERR_INVALID, "moe_align: null pointer");
+  return launch_moe_align(topk_ids, num_ids, num_experts, tile_m, sorted_token_ids, sorted_expert_ids,
+                          num_slots_out, max_slots, (hipStream_t)stream);
+}
+
+int mx_quantize(const mx_tensor* x, mx_tensor* xq, mx_tensor* scale, int32_t scale_mode, void* stream) {
+  if (int rc = check_tensor(x, "x", 2, 2)) return rc;
+  if (int rc = check_tensor(xq, "xq", 2, 2)) return rc;
+  if (int rc = check_tensor(scale, "scale", 2, 2)) return rc;
+  if (x->dtype != MX_F32 && x->dtype != MX_BF16 && x->dtype != MX_F16)
+    return set_error(MX_ERR_DTYPE, "x must be MX_F32, MX_BF16 or MX_F16");
+  if (!is_elem(xq->dtype)) return set_error(MX_ERR_DTYPE, "xq must be an MX element format");
+  if (scale->dtype != MX_E8M0) return set_error(MX_ERR_DTYPE, "scale must be MX_E8M0");
+  if (scale_mode != 0 && scale_mode != 1) return set_error(MX_ERR_INVALID, "scale_mode must be 0 (ceil) or 1 (floor)");
+  const int64_t rows = x->shape[0], K = x->shape[1];
+  if (K < 32)
+    return set_error(MX_ERR_SHAPE,
+                     "The requested block size 32 is larger than the inner most dimension of the input tensor %lld",
+                     (long long)K);
+  const int64_t Kpad = (K + 31) / 32 * 32;
+  if (xq->shape[0] != rows || xq->shape[1] != Kpad || scale->shape[0] != rows || scale->shape[1] != Kpad / 32)
+    return set_error(MX_ERR_SHAPE, "xq must be [rows, %lld] and scale [rows, %lld]", (long long)Kpad,
+                     (long long)(Kpad / 32));
+  if (x->stride[1] != 1 || xq->stride[1] != 1 || scale->stride[1] != 1)
+    return set_error(MX_ERR_LAYOUT, "x, xq and scale must be contiguous along the last axis");
+  if (xq->dtype == MX_E2M1 && xq->packed_dim != 1) return set_error(MX_ERR_LAYOUT, "xq must be packed along K");
+  QuantArgs q = {};
+  q.x = x->ptr; q.xq = (uint8_t*)xq->ptr; q.scale = (uint8_t*)scale->ptr;
+  q.rows = rows; q.K = K; q.Kpad = Kpad;
+  q.x_ld = x->stride[0]; q.xq_ld = xq->stride[0]; q.sc_ld = scale->stride[0];
+  q.x_dtype = x->dtype; q.fmt = xq->dtype; q.scale_mode = scale_mode;
+  return launch_quantize(q, (hipStream_t)stream);
+}
+
+}  // extern "C"

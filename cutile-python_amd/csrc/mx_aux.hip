@@ -1,0 +1,317 @@
+// Memory-bound helpers around the block-scaled GEMM: MX quantisation, native scale re-layout and the
+// MoE slot alignment.  All integer / byte work; results must be bit-exact.
+#include "mx_common.h"
+
+namespace mx {
+namespace {
+
+// ================================================================================================
+// MX quantiser (replaces the torch-op chain of block_quantize, test/kernels/kernel_utils.py:38-80)
+// ================================================================================================
+// Element conversion is done on the bit pattern: value = sig * 2^(ex-150) is divided by the block
+// scale 2^se by subtracting exponents, then rounded to nearest even onto the target grid in one step.
+// No floating-point operation is involved, so denormal modes and fused operations cannot change a bit.
+
+struct Unpacked {
+  uint32_t sig;   // 24-bit significand with the leading one at bit 23 (0 for zero)
+  int ex;         // biased exponent such that value = sig * 2^(ex - 150)
+  uint32_t sign;  // 0 or 1
+  int cls;        // 0 finite, 1 inf, 2 nan
+};
+
+__device__ inline Unpacked unpack_f32(uint32_t bits) {
+  Unpacked u;
+  u.sign = bits >> 31;
+  const uint32_t a = bits & 0x7FFFFFFFu;
+  u.cls = a > 0x7F800000u ? 2 : (a == 0x7F800000u ? 1 : 0);
+  int ex = (int)(a >> 23);
+  uint32_t sig = a & 0x7FFFFFu;
+  if (ex == 0) {
+    if (sig != 0) {  // subnormal: normalise
+      const int lz = __builtin_clz(sig) - 8;
+      sig <<= lz;
+      ex = 1 - lz;
+    }
+  } else {
+    sig |= 0x800000u;
+  }
+  u.sig = sig;
+  u.ex = ex;
+  return u;
+}
+
+// round-to-nearest-even of sig / 2^sh, sh in [1, 31]
+__device__ inline uint32_t rne_shift(uint32_t sig, int sh) {
+  return (sig + ((1u << (sh - 1)) - 1u) + ((sig >> sh) & 1u)) >> sh;
+}
+
+// Generic minifloat encoder: MBITS mantissa bits, minimum normal exponent EMIN, exponent bias BIAS.
+// Returns the magnitude code without clamping (may exceed the format's largest finite code).
+template <int MBITS, int EMIN, int BIAS>
+__device__ inline uint32_t encode_mag(const Unpacked& u, int se) {
+  if (u.sig == 0) return 0;
+  const int E = u.ex - 127 - se;            // exponent of x / 2^se
+  const int Eq = E > EMIN ? E : EMIN;
+  int sh = (23 - MBITS) + (Eq - E);
+  if (sh > 31) sh = 31;                     // anything this small rounds to zero
+  const uint32_t n = rne_shift(u.sig, sh);  // in units of 2^(Eq - MBITS); normal range: [2^MBITS, 2^(MBITS+1)]
+  if (E > 300) return 0xFFFFu;              // cannot happen for finite fp32 / E8M0 scales; keeps shifts sane
+  return (uint32_t)((Eq + BIAS - 1) << MBITS) + n;
+}
+
+__device__ inline uint32_t encode_e4m3(const Unpacked& u, int se, bool saturate) {
+  const uint32_t s = u.sign << 7;
+  if (u.cls == 2) return s | 0x7F;
+  if (u.cls == 1) return s | (saturate ? 0x7Eu : 0x7Fu);
+  uint32_t c = encode_mag<3, -6, 7>(u, se);
+  if (c > 0x7E) c = saturate ? 0x7E : 0x7F;   // torch's cast: above 448 after rounding -> NaN
+  return s | c;
+}
+
+__device__ inline uint32_t encode_e5m2(const Unpacked& u, int se, bool saturate) {
+  const uint32_t s = u.sign << 7;
+  if (u.cls == 2) return s | 0x7F;
+  if (u.cls == 1) return s | (saturate ? 0x7Bu : 0x7Cu);
+  uint32_t c = encode_mag<2, -14, 15>(u, se);
+  if (c > 0x7B) c = saturate ? 0x7B : 0x7C;   // IEEE-like: overflow -> inf
+  return s | c;
+}
+
+__device__ inline uint32_t encode_e2m1(const Unpacked& u, int se) {
+  const uint32_t s = u.sign << 3;
+  if (u.cls != 0) return s | 7;
+  uint32_t c = encode_mag<1, 0, 1>(u, se);
+  if (c > 7) c = 7;                           // finite-only format: clamp to +-6
+  return s | c;
+}
+
+__device__ inline float load_as_f32(const void* p, int64_t i, int dtype) {
+  if (dtype == MX_F32) return ((const float*)p)[i];
+  if (dtype == MX_BF16) return bf16_to_f32(((const uint16_t*)p)[i]);
+  return (float)((const _Float16*)p)[i];
+}
+
+// 8 lanes per 32-element block, 4 consecutive elements per lane.
+__global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
+  const int64_t KB = q.Kpad / 32;
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t blk = gid >> 3;
+  const int sub = (int)(gid & 7);
+  const bool live = blk < q.rows * KB;
+  const int64_t row = live ? blk / KB : 0, kb = live ? blk % KB : 0;
+  const int64_t k0 = kb * 32 + sub * 4;
+
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  if (live) {
+    const int64_t base = row * q.x_ld + k0;
+    if (q.x_dtype == MX_F32 && k0 + 3 < q.K && ((((uintptr_t)q.x) | (uintptr_t)(q.x_ld * 4)) & 15) == 0) {
+      const v4f t = *(const v4f*)((const float*)q.x + base);
+      v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else {
+      for (int e = 0; e < 4; ++e)
+        if (k0 + e < q.K) v[e] = load_as_f32(q.x, base + e, q.x_dtype);
+    }
+  }
+  // amax over the block on |bits| (monotone in |x| for finite values; NaN patterns compare largest)
+  uint32_t bits[4], am = 0;
+  for (int e = 0; e < 4; ++e) {
+    bits[e] = __builtin_bit_cast(uint32_t, v[e]);
+    const uint32_t a = bits[e] & 0x7FFFFFFFu;
+    am = a > am ? a : am;
+  }
+  for (int d = 1; d < 8; d <<= 1) {
+    const uint32_t o = (uint32_t)__shfl_xor((int)am, d);
+    am = o > am ? o : am;
+  }
+
+  // shared exponent
+  int se;
+  if (q.scale_mode == 0) {
+    // reference rule: 2^ceil(log2(max(amax/448, 1e-12))), ceiling taken exactly on the fp32 quotient
+    float t = __fdiv_rn(__builtin_bit_cast(float, am), 448.0f);
+    t = t > 1e-12f ? t : 1e-12f;              // NaN compares false -> 1e-12, as torch.clamp(min=) does not; see below
+    const uint32_t tb = __builtin_bit_cast(uint32_t, t);
+    se = (int)(tb >> 23) - 127 + ((tb & 0x7FFFFFu) ? 1 : 0);
+  } else {
+    // OCP MX v1.0: floor(log2 amax) - emax_elem; all-zero block -> smallest scale
+    const int emax = q.fmt == MX_E4M3 ? 8 : (q.fmt == MX_E5M2 ? 15 : 2);
+    if (am == 0) {
+      se = -127;
+    } else {
+      const int ex = (int)(am >> 23);
+      const int fl = ex ? ex - 127 : (31 - __builtin_clz(am)) - 149;
+      se = fl - emax;
+    }
+  }
+  se = se < -127 ? -127 : (se > 127 ? 127 : se);
+  const bool saturate = q.scale_mode != 0;
+
+  uint32_t code[4];
+  for (int e = 0; e < 4; ++e) {
+    const Unpacked u = unpack_f32(bits[e]);
+    code[e] = q.fmt == MX_E4M3 ? encode_e4m3(u, se, saturate)
+              : q.fmt == MX_E5M2 ? encode_e5m2(u, se, saturate)
+                                 : encode_e2m1(u, se);
+  }
+  if (!live) return;
+  if (q.fmt == MX_E2M1) {
+    // low nibble = even element (test/test_mma_scaled.py:155-160)
+    uint8_t* out = q.xq + row * q.xq_ld + (k0 >> 1);
+    out[0] = (uint8_t)(code[0] | (code[1] << 4));
+    out[1] = (uint8_t)(code[2] | (code[3] << 4));
+  } else {
+    uint8_t* out = q.xq + row * q.xq_ld + k0;
+    if (((((uintptr_t)q.xq) | (uintptr_t)q.xq_ld) & 3) == 0) {
+      *(uint32_t*)out = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
+    } else {
+      for (int e = 0; e < 4; ++e) out[e] = (uint8_t)code[e];
+    }
+  }
+  if (sub == 0) q.scale[row * q.sc_ld + kb] = (uint8_t)(se + 127);
+}
+
+// ================================================================================================
+// Native scale re-layout (see mx_common.h for the layout)
+// ================================================================================================
+__global__ __launch_bounds__(256) void pack_scales_kernel(const PackArgs p) {
+  const int64_t KB = p.K / 32;
+  const int64_t KQ = packed_scale_quads(p.K);
+  const int64_t per_batch = packed_scale_dwords(p.rows, p.K);
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= per_batch) return;
+  const int64_t b = blockIdx.y;
+  const int i4 = (int)(idx & 3), lane = (int)((idx >> 2) & 63);
+  const int64_t Q = (idx >> 8) % KQ, t64 = (idx >> 8) / KQ;
+  const int64_t row = t64 * 64 + i4 * 16 + (lane & 15);
+  const int g = lane >> 4;
+
+  int64_t srow = row;
+  bool ok = row < p.rows;
+  if (p.gather_ids) {
+    const int id = ok ? p.gather_ids[row] : -1;
+    ok = ok && id >= 0 && id < p.num_valid_ids;
+    srow = id / p.replicas;
+  }
+  uint32_t out = 0;
+  for (int t = 0; t < 4; ++t) {
+    const int64_t kb = (Q * 4 + t) * 4 + g;
+    uint32_t byte = 127;  // 1.0 for padding: multiplies zero-filled operand data
+    if (ok && kb < KB) {
+      int64_t off;
+      if (p.layout == MX_SCALE_SWIZZLE_32_4_4) {
+        const int64_t m0 = srow >> 7, m2 = (srow & 127) >> 5, m1 = srow & 31, k0 = kb >> 2, k1 = kb & 3;
+        off = ((m0 * (KB >> 2) + k0) * 32 + m1) * 16 + m2 * 4 + k1;
+      } else {
+        off = srow * p.s_row + kb * p.s_kb;
+      }
+      byte = p.src[b * p.s_batch + off];
+    }
+    out |= byte << (8 * t);
+  }
+  p.dst[b * per_batch + idx] = out;
+}
+
+// ================================================================================================
+// MoE slot alignment (replaces moe_align_tile_size_torch, test/kernels/fused_moe.py:113-173)
+// ================================================================================================
+// One workgroup.  Phase 1: histogram of expert ids.  Phase 2: exclusive scan of the per-expert block
+// counts.  Phase 3: wave 0 walks the ids in order, 64 at a time, and places each at
+// start[expert] + (number of earlier ids of that expert): a stable counting sort.
+__global__ __launch_bounds__(256) void moe_align_kernel(const int32_t* __restrict__ topk_ids, int64_t n,
+                                                        int32_t E, int32_t tile_m,
+                                                        int32_t* __restrict__ sorted_ids,
+                                                        int32_t* __restrict__ expert_ids,
+                                                        int32_t* __restrict__ num_slots_out,
+                                                        int64_t max_slots) {
+  extern __shared__ int32_t sh[];
+  int32_t* cnt = sh;          // [E] counts, then running write cursor
+  int32_t* start = sh + E;    // [E + 1] first slot of each expert
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += 256) cnt[e] = 0;
+  for (int64_t i = tid; i < max_slots; i += 256) sorted_ids[i] = (int32_t)n;
+  __syncthreads();
+  for (int64_t i = tid; i < n; i += 256) {
+    const int e = topk_ids[i];
+    if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int32_t s = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = s;
+      s += (cnt[e] + tile_m - 1) / tile_m * tile_m;
+    }
+    start[E] = s;
+    if (num_slots_out) *num_slots_out = s;
+  }
+  __syncthreads();
+  // block -> expert map; trailing unused blocks name expert 0 (their slots hold the sentinel)
+  const int64_t max_blocks = max_slots / tile_m;
+  for (int64_t blk = tid; blk < max_blocks; blk += 256) expert_ids[blk] = 0;
+  __syncthreads();
+  for (int e = tid; e < E; e += 256) {
+    for (int32_t s = start[e]; s < start[e + 1]; s += tile_m) expert_ids[s / tile_m] = e;
+    cnt[e] = start[e];  // becomes the write cursor
+  }
+  __syncthreads();
+  if (tid < 64) {
+    for (int64_t base = 0; base < n; base += 64) {
+      const int64_t i = base + tid;
+      int e = i < n ? topk_ids[i] : -1;
+      if (e >= E) e = -1;
+      bool todo = e >= 0;
+      while (__any(todo)) {
+        const uint64_t pending = __ballot(todo);
+        const int leader = __builtin_ctzll(pending);
+        const int e0 = __shfl(e, leader);
+        const bool mine = todo && e == e0;
+        const uint64_t same = __ballot(mine);
+        if (mine) {
+          const int rank = __builtin_popcountll(same & ((1ull << tid) - 1ull));
+          sorted_ids[cnt[e0] + rank] = (int32_t)i;
+          todo = false;
+        }
+        if (tid == leader) cnt[e0] += __builtin_popcountll(same);
+        // wave-synchronous: the next iteration's reads of cnt[] follow this write in program order
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+      }
+    }
+  }
+}
+
+}  // namespace
+
+int launch_quantize(const QuantArgs& q, hipStream_t stream) {
+  const int64_t threads = q.rows * (q.Kpad / 32) * 8;
+  if (threads <= 0) return MX_OK;
+  const int64_t blocks = (threads + 255) / 256;
+  if (blocks > 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "quantize: tensor too large");
+  hipLaunchKernelGGL(quantize_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, q);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "quantize_kernel launch: %s", hipGetErrorString(e));
+  return MX_OK;
+}
+
+int launch_pack_scales(const PackArgs& p, hipStream_t stream) {
+  const int64_t per_batch = packed_scale_dwords(p.rows, p.K);
+  if (per_batch <= 0 || p.batch <= 0) return MX_OK;
+  dim3 grid((unsigned)((per_batch + 255) / 256), (unsigned)p.batch);
+  hipLaunchKernelGGL(pack_scales_kernel, grid, dim3(256), 0, stream, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "pack_scales_kernel launch: %s", hipGetErrorString(e));
+  return MX_OK;
+}
+
+int launch_moe_align(const int32_t* topk_ids, int64_t num_ids, int32_t num_experts, int32_t tile_m,
+                     int32_t* sorted_token_ids, int32_t* sorted_expert_ids, int32_t* num_slots_out,
+                     int64_t max_slots, hipStream_t stream) {
+  const size_t lds = (size_t)(2 * num_experts + 1) * sizeof(int32_t);
+  if (lds > 60000) return set_error(MX_ERR_SHAPE, "moe_align: too many experts (%d)", num_experts);
+  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(256), lds, stream, topk_ids, num_ids, num_experts,
+                     tile_m, sorted_token_ids, sorted_expert_ids, num_slots_out, max_slots);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "moe_align_kernel launch: %s", hipGetErrorString(e));
+  return MX_OK;
+}
+
+}  // namespace mx

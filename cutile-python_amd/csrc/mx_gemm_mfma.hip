@@ -1,0 +1,362 @@
+// Block-scaled GEMM on the CDNA4 scaled-MFMA instruction (gfx950).
+//
+//   C[m, n] (+)= sum_k A[m, k] * As[m, k/32] * B[n, k] * Bs[n, k/32]
+//
+// A is [M][K] and B is [N][K], both K-contiguous (B is the column-major K x N operand of the
+// reference's block_scaled_matmul_kernel, test/kernels/scaled_matmul.py:12-114).  Scales arrive in
+// the native layout described in mx_common.h.
+//
+// Data path per workgroup (one BM x BN tile of C):
+//   global --(buffer_load_dwordx4 ... lds, no VGPR staging)--> LDS, two stages
+//   LDS --(ds_read_b128, XOR-swizzled 16-byte chunks, conflict free)--> VGPR fragments
+//   v_mfma_scale_f32_16x16x128_f8f6f4 with the E8M0 scales of the lane's 32-element K block taken
+//   from a VGPR byte selected by op_sel; fp32 accumulators; fused fp32/bf16 epilogue.
+//
+// MFMA operand roles: the B fragment is passed as the instruction's first matrix and the A fragment
+// as the second, so a lane ends up with four CONSECUTIVE columns n of one row m and the epilogue can
+// store 8 or 16 contiguous bytes per lane.
+//
+// K-order freedom: lane (r, g) of a 16x16x128 MFMA holds row r and the 32-element block g of the
+// K-step; its scale register byte scales exactly those 32 elements.  A and B use the same block in
+// the same lane group, so the result does not depend on which physical K positions the hardware
+// names a lane's bytes.
+#include "mx_common.h"
+
+namespace mx {
+namespace {
+
+typedef __attribute__((address_space(3))) uint8_t lds_u8;
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(3))) const v4i lds_v4i;
+
+constexpr uint32_t kOobOffset = 0x80000000u;  // beyond num_records of every descriptor we build
+
+template <int AF_, int BF_, int BM_, int BN_, int WGM_, int WGN_>
+struct Cfg {
+  static constexpr int AF = AF_, BF = BF_, BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
+  static constexpr int NW = WGM * WGN, NT = NW * 64;
+  static constexpr int A_EB = (AF == MX_E2M1) ? 4 : 8, B_EB = (BF == MX_E2M1) ? 4 : 8;
+  // MFMA K-steps (128 elements) per LDS stage: two when both operands are 4-bit so that a stage row
+  // is still 128 bytes
+  static constexpr int KSUB = (A_EB == 4 && B_EB == 4) ? 2 : 1;
+  static constexpr int BKE = 128 * KSUB;
+  static constexpr int A_RB = BKE * A_EB / 8, B_RB = BKE * B_EB / 8;   // bytes per stage row
+  static constexpr int A_CPR = A_RB / 16, B_CPR = B_RB / 16;           // 16-byte chunks per row
+  static constexpr int A_STAGE = BM * A_RB, B_STAGE = BN * B_RB, STAGE = A_STAGE + B_STAGE;
+  static constexpr int LDS_BYTES = 2 * STAGE;
+  static constexpr int A_LOADS = BM * A_CPR / NT, B_LOADS = BN * B_CPR / NT;
+  static constexpr int WTM = BM / WGM, WTN = BN / WGN;   // wave tile
+  static constexpr int MT = WTM / 16, NTL = WTN / 16;    // 16x16 MFMA tiles per wave
+  static_assert(WTM % 64 == 0 && WTN % 64 == 0, "wave tile must cover whole 64-row scale groups");
+  static_assert((BM * A_CPR) % NT == 0 && (BN * B_CPR) % NT == 0, "loads must divide evenly");
+  static_assert(A_CPR == 8 || A_CPR == 4, "row is 64 or 128 bytes");
+};
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+// swizzle term of a tile row: chunk c of row R lives at chunk position c ^ swz<CPR>(R)
+template <int CPR>
+__device__ inline int swz(int row) {
+  return (row / (16 / CPR)) % CPR;
+}
+
+// Fragment of one 16-row tile for MFMA K-step kk of the stage: 32 K elements of row `row`,
+// block gq.  8-bit formats: 32 bytes (two chunks); 4-bit: 16 bytes in the low four dwords.
+template <int RB, int EB>
+__device__ inline v8i load_frag(lds_u8* tile, int row, int kk, int gq, int sw) {
+  if constexpr (EB == 8) {
+    const int c = kk * 8 + 2 * gq;
+    const v4i lo = *(lds_v4i*)(tile + row * RB + ((c ^ sw) << 4));
+    const v4i hi = *(lds_v4i*)(tile + row * RB + (((c + 1) ^ sw) << 4));
+    return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  } else {
+    const int c = kk * 4 + gq;
+    const v4i lo = *(lds_v4i*)(tile + row * RB + ((c ^ sw) << 4));
+    return (v8i){lo.x, lo.y, lo.z, lo.w, 0, 0, 0, 0};
+  }
+}
+
+template <int BFMT, int AFMT, int T>
+__device__ inline v4f mfma_scaled(const v8i& bfrag, const v8i& afrag, const v4f& acc, int bscale,
+                                  int ascale) {
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bfrag, afrag, acc, BFMT, AFMT, T, bscale,
+                                                          T, ascale);
+}
+
+template <typename OutT>
+__device__ inline void store4(OutT* p, const v4f& v, bool accumulate, int nvalid, bool vec_ok);
+
+template <>
+__device__ inline void store4<float>(float* p, const v4f& v, bool accumulate, int nvalid,
+                                     bool vec_ok) {
+  if (nvalid >= 4 && vec_ok) {
+    v4f o = v;
+    if (accumulate) o += *(const v4f*)p;
+    *(v4f*)p = o;
+  } else {
+    for (int e = 0; e < 4; ++e)
+      if (e < nvalid) p[e] = accumulate ? p[e] + v[e] : v[e];
+  }
+}
+
+template <>
+__device__ inline void store4<uint16_t>(uint16_t* p, const v4f& v, bool accumulate, int nvalid,
+                                        bool vec_ok) {
+  if (nvalid >= 4 && vec_ok) {
+    v4f o = v;
+    if (accumulate) {
+      const uint2 old = *(const uint2*)p;
+      o.x += bf16_to_f32((uint16_t)old.x);
+      o.y += bf16_to_f32((uint16_t)(old.x >> 16));
+      o.z += bf16_to_f32((uint16_t)old.y);
+      o.w += bf16_to_f32((uint16_t)(old.y >> 16));
+    }
+    uint2 w;
+    w.x = (uint32_t)f32_to_bf16(o.x) | ((uint32_t)f32_to_bf16(o.y) << 16);
+    w.y = (uint32_t)f32_to_bf16(o.z) | ((uint32_t)f32_to_bf16(o.w) << 16);
+    *(uint2*)p = w;
+  } else {
+    for (int e = 0; e < 4; ++e)
+      if (e < nvalid) p[e] = f32_to_bf16(accumulate ? bf16_to_f32(p[e]) + v[e] : v[e]);
+  }
+}
+
+template <class C, typename OutT, bool GROUPED>
+__global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
+  lds_u8* const smem = (lds_u8*)smem_generic;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, gq = lane >> 4;
+  const int wm0 = (wave / C::WGN) * C::WTM, wn0 = (wave % C::WGN) * C::WTN;
+
+  // ---- tile of C owned by this workgroup: XCD-aware, then grouped along M --------------------------
+  const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
+  int tile_m, tile_n;
+  {
+    const int total = tiles_m * tiles_n;
+    const int pid = blockIdx.x;
+    // workgroup ids are dealt round-robin to the 8 XCDs (each has its own L2): give every XCD one
+    // contiguous range of the logical tile order
+    const int xcd = pid & 7, loc = pid >> 3, per = total >> 3, rem = total & 7;
+    const int lid = xcd * per + (xcd < rem ? xcd : rem) + loc;
+    constexpr int GM = 8;  // row tiles per group (test/kernels/kernel_utils.py:19-29 uses 8 too)
+    const int in_group = GM * tiles_n;
+    const int gid = lid / in_group, first_m = gid * GM;
+    const int gsz = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
+    const int in = lid % in_group;
+    tile_m = first_m + in % gsz;
+    tile_n = in / gsz;
+  }
+  const int m0 = tile_m * C::BM, n0 = tile_n * C::BN;
+
+  const int Kb_a = g.K * C::A_EB / 8, Kb_b = g.K * C::B_EB / 8;   // bytes per row
+  const int ksteps = (g.K + 127) / 128;
+  const int nstages = (ksteps + C::KSUB - 1) / C::KSUB;
+  const int KQ = (ksteps + 3) / 4;
+
+  int expert = 0;
+  if constexpr (GROUPED) expert = g.sorted_expert_ids[m0 / g.tile_m];
+
+  const uint8_t* Bbase = g.B + (GROUPED ? (int64_t)expert * g.b_expert_stride : 0);
+  const __amdgpu_buffer_rsrc_t rsA = make_rsrc(g.A, (uint32_t)(g.a_rows * g.lda));
+  const __amdgpu_buffer_rsrc_t rsB = make_rsrc(Bbase, (uint32_t)((int64_t)g.N * g.ldb));
+
+  // ---- per-thread global offsets of the 16-byte chunks this thread moves each stage -----------------
+  // load q of wave w fills LDS slots [(q*NW + w)*64, +64): slot s = (row s / CPR, position s % CPR)
+  uint32_t a_voff[C::A_LOADS], b_voff[C::B_LOADS];
+  int a_col[C::A_LOADS], b_col[C::B_LOADS];
+#pragma unroll
+  for (int q = 0; q < C::A_LOADS; ++q) {
+    const int slot = (q * C::NW + wave) * 64 + lane;
+    const int row = slot / C::A_CPR, pos = slot % C::A_CPR;
+    const int col = (pos ^ swz<C::A_CPR>(row)) * 16;
+    a_col[q] = col;
+    int64_t grow = m0 + row;
+    bool ok = grow < g.M;
+    if constexpr (GROUPED) {
+      const int id = ok ? g.sorted_token_ids[grow] : 0x7FFFFFFF;
+      ok = ok && id >= 0 && id < g.num_valid_ids;
+      grow = id / g.replicas;
+    }
+    a_voff[q] = ok ? (uint32_t)(grow * g.lda + col) : kOobOffset;
+  }
+#pragma unroll
+  for (int q = 0; q < C::B_LOADS; ++q) {
+    const int slot = (q * C::NW + wave) * 64 + lane;
+    const int row = slot / C::B_CPR, pos = slot % C::B_CPR;
+    const int col = (pos ^ swz<C::B_CPR>(row)) * 16;
+    b_col[q] = col;
+    const int64_t grow = n0 + row;
+    b_voff[q] = grow < g.N ? (uint32_t)(grow * g.ldb + col) : kOobOffset;
+  }
+
+  auto issue_stage = [&](int s, int buf) {
+    lds_u8* const abase = smem + buf * C::STAGE;
+    lds_u8* const bbase = abase + C::A_STAGE;
+    const int ka = s * C::A_RB, kb = s * C::B_RB;
+    const bool tail_a = ka + C::A_RB > Kb_a, tail_b = kb + C::B_RB > Kb_b;   // uniform
+#pragma unroll
+    for (int q = 0; q < C::A_LOADS; ++q) {
+      uint32_t v = a_voff[q];
+      if (tail_a && ka + a_col[q] >= Kb_a) v = kOobOffset;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_void*)(abase + (q * C::NW + wave) * 1024),
+                                               16, v, ka, 0, 0);
+    }
+#pragma unroll
+    for (int q = 0; q < C::B_LOADS; ++q) {
+      uint32_t v = b_voff[q];
+      if (tail_b && kb + b_col[q] >= Kb_b) v = kOobOffset;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(bbase + (q * C::NW + wave) * 1024),
+                                               16, v, kb, 0, 0);
+    }
+  };
+
+  // ---- scales: one 16-byte load per lane covers 4 row tiles x 4 K-steps ------------------------------
+  constexpr int AQ = C::MT / 4, BQ = C::NTL / 4;
+  const v4i* const as_ptr = (const v4i*)g.As + ((int64_t)((m0 + wm0) / 64) * KQ) * 64 + lane;
+  const v4i* const bs_ptr = (const v4i*)(g.Bs + (GROUPED ? (int64_t)expert * g.bs_expert_stride : 0)) +
+                            ((int64_t)((n0 + wn0) / 64) * KQ) * 64 + lane;
+  v4i sa[AQ], sb[BQ];
+  auto load_scales = [&](int Q) {
+#pragma unroll
+    for (int u = 0; u < AQ; ++u) sa[u] = as_ptr[((int64_t)u * KQ + Q) * 64];
+#pragma unroll
+    for (int u = 0; u < BQ; ++u) sb[u] = bs_ptr[((int64_t)u * KQ + Q) * 64];
+  };
+
+  v4f acc[C::MT][C::NTL];
+#pragma unroll
+  for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+    for (int j = 0; j < C::NTL; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+  const int swa = swz<C::A_CPR>(r), swb = swz<C::B_CPR>(r);
+
+  issue_stage(0, 0);
+  int buf = 0;
+  for (int Q = 0; Q < KQ; ++Q) {
+    load_scales(Q);
+#pragma unroll
+    for (int t0 = 0; t0 < 4; t0 += C::KSUB) {
+      const int s = Q * (4 / C::KSUB) + t0 / C::KSUB;
+      if (s < nstages) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this thread's LDS-DMA of stage s landed
+        __syncthreads();                      // everyone's landed; everyone left stage s-1's buffer
+        if (s + 1 < nstages) issue_stage(s + 1, buf ^ 1);
+        lds_u8* const atile = smem + buf * C::STAGE + (wm0 + r) * C::A_RB;
+        lds_u8* const btile = smem + buf * C::STAGE + C::A_STAGE + (wn0 + r) * C::B_RB;
+#pragma unroll
+        for (int kk = 0; kk < C::KSUB; ++kk) {
+          v8i bf[C::NTL];
+#pragma unroll
+          for (int j = 0; j < C::NTL; ++j)
+            bf[j] = load_frag<C::B_RB, C::B_EB>(btile, 16 * j, kk, gq, swb);
+#pragma unroll
+          for (int i = 0; i < C::MT; ++i) {
+            const v8i af = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
+#pragma unroll
+            for (int j = 0; j < C::NTL; ++j) {
+              // compile-time K-step index within the quad selects the scale byte
+              if (t0 + kk == 0)
+                acc[i][j] = mfma_scaled<C::BF, C::AF, 0>(bf[j], af, acc[i][j], sb[j / 4][j % 4], sa[i / 4][i % 4]);
+              else if (t0 + kk == 1)
+                acc[i][j] = mfma_scaled<C::BF, C::AF, 1>(bf[j], af, acc[i][j], sb[j / 4][j % 4], sa[i / 4][i % 4]);
+              else if (t0 + kk == 2)
+                acc[i][j] = mfma_scaled<C::BF, C::AF, 2>(bf[j], af, acc[i][j], sb[j / 4][j % 4], sa[i / 4][i % 4]);
+              else
+                acc[i][j] = mfma_scaled<C::BF, C::AF, 3>(bf[j], af, acc[i][j], sb[j / 4][j % 4], sa[i / 4][i % 4]);
+            }
+          }
+        }
+        buf ^= 1;
+      }
+    }
+  }
+
+  // ---- epilogue: lane (r, gq) of tile (i, j) holds C[m0+wm0+16i+r][n0+wn0+16j+4gq .. +3] -----------
+  OutT* const Cp = (OutT*)g.C;
+  const bool vec_ok = (g.ldc % 4 == 0) && (((uintptr_t)g.C) % 16 == 0);
+  const bool accumulate = g.accumulate != 0;
+#pragma unroll
+  for (int i = 0; i < C::MT; ++i) {
+    const int m = m0 + wm0 + 16 * i + r;
+    int64_t orow = m;
+    bool ok = m < g.M;
+    float w = 1.f;
+    if constexpr (GROUPED) {
+      const int id = ok ? g.sorted_token_ids[m] : 0x7FFFFFFF;
+      ok = ok && id >= 0 && id < g.num_valid_ids;
+      orow = id;
+      if (ok && g.topk_weights) w = g.topk_weights[id];
+    }
+    if (!ok) continue;
+#pragma unroll
+    for (int j = 0; j < C::NTL; ++j) {
+      const int n = n0 + wn0 + 16 * j + 4 * gq;
+      if (n >= g.N) continue;
+      v4f v = acc[i][j];
+      if constexpr (GROUPED) v *= w;
+      store4<OutT>(Cp + orow * g.ldc + n, v, accumulate, g.N - n, vec_ok);
+    }
+  }
+}
+
+template <class C, typename OutT, bool GROUPED>
+int launch_one(const GemmArgs& g, hipStream_t stream) {
+  auto kern = gemm_kernel<C, OutT, GROUPED>;
+  static int attr_done = 0;   // benign race: the attribute call is idempotent
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       C::LDS_BYTES);
+    if (e != hipSuccess)
+      return set_error(MX_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", C::LDS_BYTES,
+                       hipGetErrorString(e));
+    attr_done = 1;
+  }
+  const int64_t tiles = (int64_t)((g.M + C::BM - 1) / C::BM) * ((g.N + C::BN - 1) / C::BN);
+  if (tiles <= 0) return MX_OK;
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(C::NT), C::LDS_BYTES, stream, g);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "gemm_kernel launch: %s", hipGetErrorString(e));
+  return MX_OK;
+}
+
+template <int BM, int BN, int WGM, int WGN>
+int launch_fmt(const GemmArgs& g, hipStream_t stream) {
+  const bool grouped = g.sorted_token_ids != nullptr;
+#define MX_CASE(AFMT, BFMT)                                                                        \
+  if (g.a_fmt == AFMT && g.b_fmt == BFMT) {                                                        \
+    using C = Cfg<AFMT, BFMT, BM, BN, WGM, WGN>;                                                   \
+    if (g.c_dtype == MX_F32)                                                                       \
+      return grouped ? launch_one<C, float, true>(g, stream) : launch_one<C, float, false>(g, stream); \
+    return grouped ? launch_one<C, uint16_t, true>(g, stream)                                      \
+                   : launch_one<C, uint16_t, false>(g, stream);                                    \
+  }
+  MX_CASE(MX_E4M3, MX_E4M3)
+  MX_CASE(MX_E5M2, MX_E5M2)
+  MX_CASE(MX_E2M1, MX_E2M1)
+  MX_CASE(MX_E4M3, MX_E2M1)
+#undef MX_CASE
+  return set_error(MX_ERR_DTYPE, "MFMA kernel: unsupported element format pair (%d, %d)", g.a_fmt,
+                   g.b_fmt);
+}
+
+}  // namespace
+
+int launch_gemm_mfma(const GemmArgs& g, int kernel_id, hipStream_t stream) {
+  if (g.c_dtype != MX_F32 && g.c_dtype != MX_BF16)
+    return set_error(MX_ERR_DTYPE, "MFMA kernel: output dtype %d not supported", g.c_dtype);
+  switch (kernel_id) {
+    case MX_KERNEL_MFMA_128x128: return launch_fmt<128, 128, 2, 2>(g, stream);
+    case MX_KERNEL_MFMA_256x256: return launch_fmt<256, 256, 2, 4>(g, stream);
+    case MX_KERNEL_MFMA_256x256_W4: return launch_fmt<256, 256, 2, 2>(g, stream);
+  }
+  return set_error(MX_ERR_INVALID, "unknown MFMA kernel id %d", kernel_id);
+}
+
+}  // namespace mx

@@ -1,0 +1,203 @@
+/*
+ * mxgemm.h -- C ABI of libmxgemm.so: block-scaled (MX) matrix multiply for AMD MI355X (gfx950).
+ *
+ * Plain C, plain pointers and sizes; no C++ or framework types cross this boundary.  Every entry
+ * point enqueues work on the given hipStream_t (passed as void*; NULL = the null stream) and
+ * returns without synchronising.  Return value: 0 on success, a negative MX_ERR_* otherwise; the
+ * message of the last error on the calling thread is available from mx_last_error().
+ * The library keeps no mutable global state besides that thread-local string, so calls from
+ * several host threads are safe.  Nothing here allocates device memory: any workspace is passed
+ * in by the caller.
+ *
+ * Each declaration names the reference interface (NVIDIA cuTile Python, path:line) it stands in for.
+ */
+#ifndef MXGEMM_H
+#define MXGEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MXGEMM_VERSION 100
+
+/* Exported symbols (the library is built with hidden default visibility). */
+#if defined(__GNUC__)
+#define MX_API __attribute__((visibility("default")))
+#else
+#define MX_API
+#endif
+
+/* Error codes. */
+enum {
+  MX_OK = 0,
+  MX_ERR_INVALID = -1,      /* bad argument (null pointer, rank, negative stride ...)            */
+  MX_ERR_SHAPE = -2,        /* shapes of operands / scales / output do not agree                 */
+  MX_ERR_DTYPE = -3,        /* unsupported dtype or dtype combination                            */
+  MX_ERR_LAYOUT = -4,       /* layout not supported by the requested kernel                      */
+  MX_ERR_WORKSPACE = -5,    /* workspace missing or too small                                    */
+  MX_ERR_DEVICE = -6,       /* no gfx950 device / HIP error                                      */
+  MX_ERR_LAUNCH = -7        /* kernel launch failed                                              */
+};
+
+/* Element / scale / output type codes.  The three element formats use the codes the CDNA4
+ * v_mfma_scale_f32_*_f8f6f4 instruction uses for its cbsz/blgp fields. */
+enum {
+  MX_E4M3 = 0,   /* float8_e4m3fn, 1 byte                                            */
+  MX_E5M2 = 1,   /* float8_e5m2,   1 byte                                            */
+  MX_E2M1 = 4,   /* float4_e2m1fn, two per byte, low nibble = even logical element   */
+  MX_E8M0 = 8,   /* float8_e8m0fnu scale byte, value 2^(b-127), 0xFF = NaN           */
+  MX_F32 = 16,
+  MX_BF16 = 17,
+  MX_F16 = 18,
+  MX_I32 = 24
+};
+
+/*
+ * Tensor descriptor: pointer + logical shape + strides.  Mirrors the per-array words the
+ * reference's launcher passes to a kernel (ptr, shape[ndim], stride[ndim];
+ * cext/tile_kernel.cpp:1883-1917, 1999-2002).
+ *   shape[]  -- LOGICAL element counts (for MX_E2M1: number of 4-bit elements).
+ *   stride[] -- in units of the storage type: bytes for all 8- and 4-bit formats, elements for
+ *               f32/bf16/i32.  For MX_E2M1 exactly one dimension is the packed one: it has stride 1
+ *               and holds two logical elements per byte; `packed_dim` names it.
+ */
+typedef struct mx_tensor {
+  void* ptr;
+  int32_t dtype;
+  int32_t ndim;          /* 1..4 */
+  int64_t shape[4];
+  int64_t stride[4];
+  int32_t packed_dim;    /* MX_E2M1 only: index of the dimension packed two-per-byte; else -1 */
+  int32_t reserved;
+} mx_tensor;
+
+/* Scale tensor layouts accepted by mx_gemm / mx_gemm_grouped. */
+enum {
+  MX_SCALE_2D = 0,        /* logical [rows, K/B] (A) or [K/B, cols] (B), any strides
+                             (samples/BlockScaledMatMul.py:243-250)                              */
+  MX_SCALE_SWIZZLE_32_4_4 = 1, /* contiguous [rows/128, (K/B)/4, 32, 16] as produced by
+                             swizzle_32_4_4 (test/kernels/kernel_utils.py:83-98); for B the rows
+                             are the N index                                                      */
+  MX_SCALE_NATIVE = 2     /* this library's MFMA-ready layout written by mx_pack_scales          */
+};
+
+/* Kernel selection. */
+enum {
+  MX_KERNEL_AUTO = 0,
+  MX_KERNEL_GENERIC = 1,      /* one thread per output element; any strides / packing / block  */
+  MX_KERNEL_MFMA_128x128 = 2, /* v_mfma_scale tiles, 128x128 macro tile, 4 waves                */
+  MX_KERNEL_MFMA_256x256 = 3, /* 256x256 macro tile, 8 waves                                    */
+  MX_KERNEL_MFMA_256x256_W4 = 4, /* 256x256 macro tile, 4 waves                                 */
+  MX_KERNEL_DECODE = 5        /* skinny-M (M <= 32) weight-streaming kernel                     */
+};
+
+typedef struct mx_gemm_opts {
+  int32_t struct_size;    /* sizeof(mx_gemm_opts), for forward compatibility                    */
+  int32_t accumulate;     /* 0: C = A@B ; 1: C = A@B + C  (the `acc` operand of ct.mma_scaled)   */
+  int32_t a_scale_layout; /* MX_SCALE_*                                                          */
+  int32_t b_scale_layout;
+  int32_t kernel;         /* MX_KERNEL_*                                                         */
+  int32_t block_size;     /* scaling block size B along K: 32 (16 only with MX_KERNEL_GENERIC)   */
+  int32_t reserved[2];
+} mx_gemm_opts;
+
+/* Library version (MXGEMM_VERSION of the built library). */
+MX_API int mx_version(void);
+
+/* Message of the last error raised on the calling thread ("" if none).
+ * Stands in for the Python exception text of cext/tile_kernel.cpp:3910-3916. */
+MX_API const char* mx_last_error(void);
+
+/* Returns 0 if the current HIP device is a gfx950 part, MX_ERR_DEVICE otherwise.
+ * (reference: get_compute_capability gate, samples/BlockScaledMatMul.py:308-311.) */
+MX_API int mx_device_check(void);
+
+/*
+ * Bytes of device workspace mx_gemm needs for the given problem (native re-layout of the scale
+ * tensors).  0 if both scale tensors are already MX_SCALE_NATIVE or the generic kernel is used.
+ */
+MX_API int64_t mx_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, const mx_gemm_opts* opts);
+
+/*
+ * C[M,N] (+)= sum_k A[m,k]*As[m,k/B] * B[k,n]*Bs[k/B,n]   with fp32 accumulation.
+ * Replaces: ct.launch(stream, grid, block_scaled_matmul_kernel, (A, A_scale, B, B_scale, C, tm, tn,
+ * tk, scaling_block_size))  -- samples/BlockScaledMatMul.py:294-295, kernel
+ * test/kernels/scaled_matmul.py:12-114, op semantics src/cuda/tile/_stub.py:2198-2235.
+ *   A  [M,K]  MX_E4M3 | MX_E5M2 | MX_E2M1        As [M,K/B] MX_E8M0 (or 4-D swizzled / native)
+ *   B  [K,N]  same family (formats may differ)    Bs [K/B,N]
+ *   C  [M,N]  MX_F32 | MX_BF16
+ * The MFMA kernels need K-contiguous A (stride[1]==1) and B (stride[0]==1), 16-byte aligned rows
+ * and block_size 32; MX_KERNEL_AUTO falls back to the generic kernel otherwise.
+ * Optional leading batch dimension (ndim 3) is handled by the generic kernel with broadcast of
+ * size-1 batches (test/test_mma_scaled.py:128-145).
+ */
+MX_API int mx_gemm(const mx_tensor* A, const mx_tensor* A_scale, const mx_tensor* B,
+            const mx_tensor* B_scale, mx_tensor* C, const mx_gemm_opts* opts, void* workspace,
+            int64_t workspace_bytes, void* stream);
+
+/*
+ * Grouped (MoE) variant.  Replaces: ct.launch(..., fused_moe_kernel, (A, B, C, topk_weights,
+ * sorted_token_ids, sorted_expert_ids, num_token_replicas, mul_routed_weight, TILE_M, TILE_N,
+ * TILE_K)) -- samples/MoE.py:338-375, kernel test/kernels/fused_moe.py:14-82, with the bf16 ct.mma
+ * replaced by the block-scaled product.
+ *   A  [T,K] tokens, As [T,K/32];  W [E,N,K] (K contiguous), Ws [E,N,K/32];  C [T*replicas? ,N]:
+ *   for every slot p of sorted_token_ids with id = sorted_token_ids[p] < num_valid_ids:
+ *       C[id,:] = (A[id / num_token_replicas,:] * As) @ (W[e,:,:] * Ws[e]).T * (w ? w[id] : 1)
+ *   where e = sorted_expert_ids[p / tile_m].  Slots holding the sentinel are skipped.
+ *   topk_weights may be NULL (no routed-weight multiply).
+ * Workspace: mx_gemm_grouped_workspace_bytes().
+ */
+MX_API int64_t mx_gemm_grouped_workspace_bytes(int64_t num_slots, int64_t N, int64_t K, int64_t E,
+                                        const mx_gemm_opts* opts);
+MX_API int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* A_scale, const mx_tensor* W,
+                    const mx_tensor* W_scale, mx_tensor* C, const float* topk_weights,
+                    const int32_t* sorted_token_ids, int64_t num_slots,
+                    const int32_t* sorted_expert_ids, int32_t tile_m, int32_t num_token_replicas,
+                    int64_t num_valid_ids, const mx_gemm_opts* opts, void* workspace,
+                    int64_t workspace_bytes, void* stream);
+
+/*
+ * Device-side replacement of moe_align_tile_size_torch (test/kernels/fused_moe.py:113-173): stable
+ * counting sort of the flattened expert ids, each expert padded to a multiple of tile_m with the
+ * sentinel value num_ids.  Outputs must hold mx_moe_align_max_slots(num_ids, num_experts, tile_m)
+ * int32 slots and that number / tile_m blocks; unused trailing slots are filled with the sentinel
+ * and unused trailing blocks with expert 0.  *num_slots_out (device int32, optional) receives the
+ * number of slots actually used.  No host synchronisation.
+ */
+MX_API int64_t mx_moe_align_max_slots(int64_t num_ids, int32_t num_experts, int32_t tile_m);
+MX_API int mx_moe_align(const int32_t* topk_ids, int64_t num_ids, int32_t num_experts, int32_t tile_m,
+                 int32_t* sorted_token_ids, int32_t* sorted_expert_ids, int32_t* num_slots_out,
+                 void* stream);
+
+/*
+ * MX quantisation of the last axis in blocks of 32 (replaces the torch-op sequence of
+ * block_quantize, test/kernels/kernel_utils.py:38-80).
+ *   x      [rows, K] MX_F32 | MX_BF16 | MX_F16, last stride 1
+ *   xq     [rows, Kpad] MX_E4M3 | MX_E5M2 (1 byte each) or MX_E2M1 (packed along K), Kpad = K
+ *          rounded up to 32 (tail zero-padded as the reference does)
+ *   scale  [rows, Kpad/32] MX_E8M0
+ *   scale_mode 0 = "ceil":  2^ceil(log2(max(amax/448, 1e-12))), non-saturating element cast
+ *              1 = "floor": 2^(floor(log2 amax) - emax_elem), saturating element cast (OCP MX v1.0)
+ */
+MX_API int mx_quantize(const mx_tensor* x, mx_tensor* xq, mx_tensor* scale, int32_t scale_mode,
+                void* stream);
+
+/*
+ * Re-lays a scale tensor into the MFMA-ready native layout consumed by the MFMA kernels
+ * (no reference counterpart: the reference's swizzle_32_4_4, test/kernels/kernel_utils.py:83-98,
+ * is the Blackwell analogue).  `scale` is [rows, K/32] logical with any strides (MX_SCALE_2D; pass a
+ * transposed descriptor for a [K/32, cols] tensor), or the contiguous 4-D swizzled tensor
+ * (MX_SCALE_SWIZZLE_32_4_4); an optional leading batch dimension (experts) is kept.
+ * `packed` must hold mx_packed_scale_bytes(rows, K) bytes per batch entry.
+ */
+MX_API int64_t mx_packed_scale_bytes(int64_t rows, int64_t K);
+MX_API int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, void* packed,
+                   void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXGEMM_H */

@@ -1,0 +1,103 @@
+"""GPU parity of the skinny-M weight-streaming kernel and of the grouped (MoE) GEMM."""
+import numpy as np
+import pytest
+import torch
+
+from mxutil import oracle_matmul, randn_operand
+from oracle import mx_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("M,N,K", [(32, 256, 1024), (7, 1792, 2048), (16, 48, 512), (32, 4096, 8192), (1, 16, 4096)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=str)
+def test_decode_kernel(ct, dev, M, N, K, out_dtype):
+    x = randn_operand(M, K, O.E4M3, 81, dev)
+    w = randn_operand(N, K, O.E2M1, 82, dev, std=0.02)
+    ref = oracle_matmul(x, w)
+    c = ct.block_scaled_matmul(x.storage, x.scale_t, w.storage.T, w.scale_t.T, b_format="e2m1",
+                               out_dtype=out_dtype, kernel="decode")
+    err = O.rel_fro(c.float().cpu(), ref)
+    print(f"decode {M}x{N}x{K} {out_dtype} rel_fro={err:.3e}", flush=True)
+    assert err <= (1e-3 if out_dtype == torch.float32 else 8e-3)
+    # the automatic choice for this shape family is the same kernel
+    c2 = ct.block_scaled_matmul(x.storage, x.scale_t, w.storage.T, w.scale_t.T, b_format="e2m1",
+                                out_dtype=out_dtype)
+    assert torch.equal(c, c2)
+    # and the tiled MFMA kernel agrees within tolerance
+    c3 = ct.block_scaled_matmul(x.storage, x.scale_t, w.storage.T, w.scale_t.T, b_format="e2m1",
+                                out_dtype=out_dtype, kernel="mfma128")
+    assert O.rel_fro(c3.float().cpu(), ref) <= (1e-3 if out_dtype == torch.float32 else 8e-3)
+
+
+def test_decode_accumulate(ct, dev):
+    x = randn_operand(32, 1024, O.E4M3, 83, dev)
+    w = randn_operand(64, 1024, O.E2M1, 84, dev)
+    z = torch.randn((32, 64), generator=torch.Generator().manual_seed(85))
+    acc = z.to(dev)
+    ct.block_scaled_matmul(x.storage, x.scale_t, w.storage.T, w.scale_t.T, b_format="e2m1", C=acc,
+                           accumulate=True, kernel="decode")
+    assert O.rel_fro(acc.cpu(), oracle_matmul(x, w) + z) < 1e-3
+
+
+@pytest.mark.parametrize("T,topk,E,tile", [(7, 2, 4, 4), (48, 8, 64, 16), (5, 1, 8, 128), (4096, 2, 8, 256),
+                                           (110, 4, 16, 128), (256, 6, 1408, 128)])
+def test_moe_align_matches_oracle(ct, dev, T, topk, E, tile):
+    """test/kernels/fused_moe.py:113-173; shapes from samples/MoE.py:420-462 and test/bench_moe.py:16-24."""
+    g = torch.Generator().manual_seed(T + E)
+    ids = torch.topk(torch.rand((T, E), generator=g), topk, dim=1).indices
+    want_ids, want_e = O.moe_align_tile_size(ids.numpy(), tile, E)
+    got_ids, got_e = ct.moe_align_tile_size(ids.to(dev), tile, E)
+    assert got_ids.dtype == torch.int32 and got_e.dtype == torch.int32
+    assert np.array_equal(got_ids.cpu().numpy(), want_ids)
+    assert np.array_equal(got_e.cpu().numpy(), want_e)
+    # without the trim nothing synchronises; the tail is sentinel / expert 0
+    all_ids, all_e = ct.moe_align_tile_size(ids.to(dev), tile, E, exact=False)
+    assert np.array_equal(all_ids[:len(want_ids)].cpu().numpy(), want_ids)
+    assert bool((all_ids[len(want_ids):] == T * topk).all()) and bool((all_e[len(want_e):] == 0).all())
+
+
+def _moe_case(T, K, N, E, topk, seed, dev, w_std=0.1):
+    a = randn_operand(T, K, O.E4M3, seed, dev, std=0.5)
+    w = randn_operand(E * N, K, O.E4M3, seed + 1, dev, std=w_std)
+    g = torch.Generator().manual_seed(seed + 2)
+    ids = torch.topk(torch.rand((T, E), generator=g), topk, dim=1).indices
+    ref = O.grouped_reference(a.codes, a.scales, w.codes.reshape(E, N, K), w.scales.reshape(E, N, K // 32),
+                              ids.numpy())
+    W = w.storage.view(E, N, K)
+    Ws = w.scale_t.view(E, N, K // 32)
+    return a, W, Ws, ids, ref
+
+
+@pytest.mark.parametrize("kernel,tile", [("generic", 16), ("generic", 128), ("mfma128", 128), ("mfma128", 256),
+                                         ("mfma256", 256), ("mfma256w4", 256), ("auto", 128), ("auto", 256)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=str)
+def test_grouped_gemm_sample_shape(ct, dev, kernel, tile, out_dtype):
+    """samples/MoE.py:420-462 shape: 48 tokens, hidden 512, 64 experts, top-8; N = 1024."""
+    T, K, N, E, topk = 48, 512, 1024, 64, 8
+    a, W, Ws, ids, ref = _moe_case(T, K, N, E, topk, 91, dev)
+    sid, eid = ct.moe_align_tile_size(ids.to(dev), tile, E)
+    C = torch.full((T, topk, N), float("nan"), device=dev, dtype=out_dtype)
+    ct.invoke_fused_moe_scaled(a.storage, a.scale_t, W, Ws, C, None, sid, eid, False, topk, tile, kernel=kernel)
+    err = O.rel_fro(C.view(-1, N).float().cpu(), ref)
+    print(f"grouped {kernel} tile={tile} {out_dtype} rel_fro={err:.3e}", flush=True)
+    assert err <= (1e-3 if out_dtype == torch.float32 else 8e-3)
+
+
+@pytest.mark.parametrize("kernel", ["generic", "mfma128", "mfma256"])
+def test_grouped_gemm_routed_weight_replicas1_and_padded_ids(ct, dev, kernel):
+    """Second GEMM of the sample: replicas = 1, rows multiplied by the routed weight
+    (test/kernels/fused_moe.py:75-77); index arrays left at their worst-case length."""
+    T, K, N, E, topk = 300, 256, 384, 8, 1
+    a, W, Ws, ids, ref = _moe_case(T, K, N, E, topk, 95, dev)
+    wts = torch.rand((T, topk), generator=torch.Generator().manual_seed(96))
+    sid, eid = ct.moe_align_tile_size(ids.to(dev), 256, E, exact=False)
+    C = torch.zeros((T * topk, N), device=dev, dtype=torch.float32)
+    ct.invoke_fused_moe_scaled(a.storage, a.scale_t, W, Ws, C, wts.to(dev), sid, eid, True, 1, 256, kernel=kernel)
+    assert O.rel_fro(C.cpu(), ref * wts.reshape(-1, 1)) < 1e-3
+    # pre-packed expert scales give the same bits
+    if kernel != "generic":
+        C2 = torch.zeros_like(C)
+        ct.invoke_fused_moe_scaled(a.storage, a.scale_t, W, ct.pack_scales(Ws), C2, wts.to(dev), sid, eid, True, 1,
+                                   256, kernel=kernel)
+        assert torch.equal(C, C2)

@@ -1,0 +1,153 @@
+"""GPU parity: the HIP block-scaled GEMM (through the C ABI) against the CPU oracle on the same
+seeded inputs.  Tolerances: relative Frobenius error <= 1e-3 (fp32 output) / 8e-3 (bf16 output)."""
+import numpy as np
+import pytest
+import torch
+
+from mxutil import Operand, oracle_matmul, randn_operand, raw_operand
+from oracle import mx_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-3, torch.bfloat16: 8e-3}
+MFMA = ["mfma128", "mfma256", "mfma256w4"]
+
+
+def _run(ct, a: Operand, b: Operand, **kw):
+    return ct.block_scaled_matmul(a.storage, a.scale_t, b.storage.T, b.scale_t.T, a_format=a.fmt_kw,
+                                  b_format=b.fmt_kw, **kw)
+
+
+def _check(c, ref, out_dtype, what=""):
+    assert c.dtype == out_dtype
+    err = O.rel_fro(c.float().cpu(), ref)
+    print(f"{what} rel_fro={err:.3e}", flush=True)
+    assert err <= TOL[out_dtype], f"{what}: relative Frobenius error {err:.3e}"
+
+
+@pytest.mark.parametrize("kernel", ["generic"] + MFMA)
+def test_known_answers(ct, dev, kernel):
+    # src/cuda/tile/_stub.py:2309-2328: 128^3 ones with all scales 2.0 -> 512.0 everywhere
+    one = torch.ones((128, 128), device=dev).to(torch.float8_e4m3fn)
+    two = torch.full((128, 4), 2.0, device=dev).to(torch.float8_e8m0fnu)
+    c = ct.block_scaled_matmul(one, two, one.T, two.T, kernel=kernel)
+    assert c.unique().tolist() == [512.0]
+
+
+def test_known_answer_small_generic(ct, dev):
+    # src/cuda/tile/_stub.py:2248-2259: ones(2x64) . ones(64x2), scales 2.0 -> 256.0
+    x = torch.ones((2, 64), device=dev).to(torch.float8_e4m3fn)
+    s = torch.full((2, 2), 2.0, device=dev).to(torch.float8_e8m0fnu)
+    z = ct.mma_scaled(x, s, x.T.contiguous(), s.T.contiguous(), torch.zeros((2, 2), device=dev))
+    assert z.tolist() == [[256.0, 256.0], [256.0, 256.0]]
+
+
+FORMATS = [(O.E4M3, O.E4M3), (O.E5M2, O.E5M2), (O.E2M1, O.E2M1), (O.E4M3, O.E2M1)]
+
+
+@pytest.mark.parametrize("kernel", MFMA)
+@pytest.mark.parametrize("fa,fb", FORMATS, ids=lambda f: str(f))
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=str)
+def test_gemm_aligned(ct, dev, kernel, fa, fb, out_dtype):
+    M, N, K = 256, 512, 1024
+    a = randn_operand(M, K, fa, 11, dev, "uniform6" if fa == O.E2M1 else "randn")
+    b = randn_operand(N, K, fb, 12, dev, "uniform6" if fb == O.E2M1 else "randn")
+    c = _run(ct, a, b, out_dtype=out_dtype, kernel=kernel)
+    _check(c, oracle_matmul(a, b), out_dtype, f"{kernel} {fa}x{fb} {out_dtype}")
+
+
+@pytest.mark.parametrize("kernel", MFMA)
+@pytest.mark.parametrize("fa,fb", FORMATS, ids=lambda f: str(f))
+@pytest.mark.parametrize("M,N,K", [(300, 200, 160), (1, 1, 32), (129, 257, 96), (64, 700, 544)])
+def test_gemm_ragged(ct, dev, kernel, fa, fb, M, N, K):
+    """Edge tiles in M and N and a K that is a multiple of 32 but not of the K tile: zero padding of
+    test/kernels/scaled_matmul.py:66-104."""
+    a = randn_operand(M, K, fa, 21, dev)
+    b = randn_operand(N, K, fb, 22, dev)
+    for out_dtype in (torch.float32, torch.bfloat16):
+        c = _run(ct, a, b, out_dtype=out_dtype, kernel=kernel)
+        _check(c, oracle_matmul(a, b), out_dtype, f"{kernel} {fa}x{fb} {M}x{N}x{K} {out_dtype}")
+
+
+@pytest.mark.parametrize("kernel", ["generic"] + MFMA)
+def test_sample_shape_rand_inputs_both_scale_layouts(ct, dev, kernel):
+    """samples/BlockScaledMatMul.py:323-364: 512x512x768, torch.rand inputs, ceil-rule quantiser, plain and
+    swizzle_32_4_4 scales, assert_close(atol=1e-4, rtol=1e-3)."""
+    a = randn_operand(512, 768, O.E4M3, 31, dev, "rand", "ceil")
+    b = randn_operand(512, 768, O.E4M3, 32, dev, "rand", "ceil")
+    ref = oracle_matmul(a, b)
+    c = ct.block_scaled_matmul(a.storage, a.scale_t, b.storage.T, b.scale_t.T, kernel=kernel)
+    torch.testing.assert_close(c.cpu(), ref, atol=1e-4, rtol=1e-3)
+    a_sw = ct.swizzle_32_4_4(a.scale_t)
+    b_sw = ct.swizzle_32_4_4(b.scale_t.T.T.contiguous())  # (N, K/32), as the sample passes it
+    c2 = ct.block_scaled_matmul(a.storage, a_sw, b.storage.T, b_sw, kernel=kernel)
+    torch.testing.assert_close(c2.cpu(), ref, atol=1e-4, rtol=1e-3)
+    assert torch.equal(c, c2)
+
+
+@pytest.mark.parametrize("kernel", MFMA)
+def test_prepacked_scales_and_accumulate(ct, dev, kernel):
+    a = randn_operand(256, 512, O.E4M3, 41, dev)
+    b = randn_operand(384, 512, O.E4M3, 42, dev)
+    ref = oracle_matmul(a, b)
+    pa, pb = ct.pack_scales(a.scale_t), ct.pack_scales(b.scale_t.T, transposed=True)
+    c = ct.block_scaled_matmul(a.storage, pa, b.storage.T, pb, kernel=kernel)
+    c_plain = _run(ct, a, b, kernel=kernel)
+    assert torch.equal(c, c_plain)
+    _check(c, ref, torch.float32, "prepacked")
+    g = torch.Generator().manual_seed(43)
+    z = torch.randn((256, 384), generator=g)
+    acc = z.to(dev)
+    out = ct.block_scaled_matmul(a.storage, a.scale_t, b.storage.T, b.scale_t.T, C=acc, accumulate=True,
+                                 kernel=kernel)
+    assert out.data_ptr() == acc.data_ptr()
+    _check(out, ref + z, torch.float32, "accumulate")
+
+
+@pytest.mark.parametrize("kernel", MFMA + ["generic"])
+def test_raw_bytes_with_nan_codes(ct, dev, kernel):
+    """test/test_mma_scaled.py:103-125 feeds raw random bytes, NaN encodings included; NaNs must propagate
+    to exactly the rows/columns the oracle says (assert_close with equal_nan)."""
+    a = raw_operand(64, 256, O.E4M3, 51, dev, allow_nan=True)
+    b = raw_operand(48, 256, O.E4M3, 52, dev, allow_nan=True)
+    ref = oracle_matmul(a, b)
+    c = _run(ct, a, b, kernel=kernel).cpu()
+    assert torch.equal(torch.isnan(c), torch.isnan(ref))
+    torch.testing.assert_close(c, ref, atol=1e-2, rtol=1e-2, equal_nan=True)
+
+
+def test_auto_dispatch_matches_explicit(ct, dev):
+    a = randn_operand(384, 1024, O.E4M3, 61, dev)
+    b = randn_operand(1536, 1024, O.E4M3, 62, dev)
+    ref = oracle_matmul(a, b)
+    _check(_run(ct, a, b), ref, torch.float32, "auto")
+    # a layout the MFMA kernels cannot take (row-major K x N operand) goes to the general kernel
+    b_rowmajor = b.storage.T.contiguous()
+    bs_rowmajor = b.scale_t.T.contiguous()
+    c = ct.block_scaled_matmul(a.storage, a.scale_t, b_rowmajor, bs_rowmajor)
+    _check(c, ref, torch.float32, "auto->generic")
+    with pytest.raises(ct.TileTypeError, match="cannot run this problem"):
+        ct.block_scaled_matmul(a.storage, a.scale_t, b_rowmajor, bs_rowmajor, kernel="mfma128")
+
+
+def test_concurrent_launch_threads(ct, dev):
+    """test/test_concurrent_launch.py:49-72: several Python threads launching at once."""
+    import threading
+    a = randn_operand(128, 256, O.E4M3, 71, dev)
+    b = randn_operand(128, 256, O.E4M3, 72, dev)
+    want = _run(ct, a, b)
+    errs = []
+
+    def work():
+        try:
+            for _ in range(50):
+                c = _run(ct, a, b)
+            torch.cuda.synchronize()
+            if not torch.equal(c, want):
+                errs.append("mismatch")
+        except Exception as e:  # noqa: BLE001
+            errs.append(repr(e))
+
+    ts = [threading.Thread(target=work) for _ in range(8)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    assert not errs, errs

@@ -1,0 +1,121 @@
+"""GPU parity of the on-device MX quantiser and the scale re-layout: bit-exact against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as O
+
+pytestmark = pytest.mark.gpu
+DT = {O.E4M3: torch.float8_e4m3fn, O.E5M2: torch.float8_e5m2, O.E2M1: "e2m1"}
+
+
+def _special_rows(K):
+    """Rows that exercise the corners: zeros, one-hot, subnormals, huge, exact powers of two, the fp32
+    log2 edge 2^k(1+2^-23), values on rounding ties."""
+    rows = []
+    z = np.zeros(K, np.float32); rows.append(z.copy())
+    r = z.copy(); r[3] = 1.0; rows.append(r)
+    r = z.copy(); r[::2] = np.float32(1e-41); r[1] = np.float32(3e-39); rows.append(r)      # subnormal inputs
+    r = z.copy(); r[:] = np.float32(3e38); r[5] = -np.float32(3.4e38); rows.append(r)       # near fp32 max
+    r = z.copy(); r[:32] = np.float32(448.0) * np.float32(2.0 ** -8) * (np.float32(1) + np.float32(2.0 ** -23)); rows.append(r)
+    r = z.copy(); r[:32] = 448.0; r[32:64] = 464.0 / 2; r[64:96] = 6.0; rows.append(r)
+    ties = np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, 7.0, 0.0625, 17.0, 18.0, 19.0, 20.0, 21.0, 22.0],
+                    np.float32)
+    r = z.copy(); r[:16] = ties; r[16:32] = -ties; r[32:48] = ties * 8; r[48:64] = ties * 2.0 ** -12; rows.append(r)
+    r = z.copy(); r[:] = np.float32(2.0 ** -126); r[7] = np.float32(2.0 ** -120); rows.append(r)
+    return np.stack(rows)
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2, O.E2M1])
+@pytest.mark.parametrize("mode", ["ceil", "floor"])
+def test_quantize_bit_exact(ct, dev, fmt, mode):
+    K = 256
+    g = torch.Generator().manual_seed(5)
+    x = torch.cat([torch.randn((61, K), generator=g), torch.randn((30, K), generator=g) * 1e-3,
+                   torch.rand((20, K), generator=g) * 12 - 6, torch.from_numpy(_special_rows(K))])
+    xq, sc = ct.block_quantize(x.to(dev), 32, DT[fmt], scale_mode=mode)
+    codes, sb = O.block_quantize(x.numpy(), 32, fmt, mode)
+    got_s = sc.view(torch.uint8).cpu().numpy()
+    assert np.array_equal(got_s, sb), np.argwhere(got_s != sb)[:10]
+    got = xq.view(torch.uint8).cpu().numpy()
+    want = O.pack_fp4(codes) if fmt == O.E2M1 else codes
+    assert got.shape == want.shape
+    bad = np.argwhere(got != want)
+    assert bad.size == 0, (bad[:10], got[tuple(bad[0])], want[tuple(bad[0])], x.numpy()[bad[0][0]].max())
+    assert sc.dtype == torch.float8_e8m0fnu and sc.shape == (x.shape[0], K // 32)
+
+
+def test_quantize_padding_3d_and_bf16(ct, dev):
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn((3, 5, 72), generator=g)          # K = 72 -> padded to 96 (kernel_utils.py:62-67)
+    xq, sc = ct.block_quantize(x.to(dev), 32)
+    codes, sb = O.block_quantize(x.numpy(), 32, O.E4M3, "ceil")
+    assert xq.shape == (3, 5, 96) and xq.dtype == torch.float8_e4m3fn and sc.shape == (3, 5, 3)
+    assert np.array_equal(xq.view(torch.uint8).cpu().numpy(), codes)
+    assert np.array_equal(sc.view(torch.uint8).cpu().numpy(), sb)
+    xb = torch.randn((33, 160), generator=g).to(torch.bfloat16)
+    xq, sc = ct.block_quantize(xb.to(dev), 32, scale_mode="floor")
+    codes, sb = O.block_quantize(xb.float().numpy(), 32, O.E4M3, "floor")
+    assert np.array_equal(xq.view(torch.uint8).cpu().numpy(), codes)
+    assert np.array_equal(sc.view(torch.uint8).cpu().numpy(), sb)
+    with pytest.raises(ValueError, match="larger than the inner most dimension"):
+        ct.block_quantize(torch.zeros((4, 16), device=dev), 32)
+
+
+def test_quantize_dequantize_roundtrip_large(ct, dev):
+    """Full benchmark-size operand (8192 x 8192): quantise on the GPU, check invariants that do not need the
+    CPU oracle at this size, and compare a 64-row sample bit-for-bit."""
+    g = torch.Generator().manual_seed(1234)
+    x = torch.randn((8192, 8192), generator=g)
+    xq, sc = ct.block_quantize(x.to(dev), 32, scale_mode="floor")
+    rows = torch.arange(0, 8192, 128)
+    codes, sb = O.block_quantize(x[rows].numpy(), 32, O.E4M3, "floor")
+    assert np.array_equal(xq[rows.to(dev)].view(torch.uint8).cpu().numpy(), codes)
+    assert np.array_equal(sc[rows.to(dev)].view(torch.uint8).cpu().numpy(), sb)
+    q = xq.view(torch.uint8)
+    assert int(((q & 0x7F) == 0x7F).sum()) == 0                       # saturating: no NaN codes
+    # idempotence: quantising the dequantised tensor with the same rule reproduces codes and scales
+    deq = xq.float() * torch.repeat_interleave(sc.float(), 32, dim=1)
+    xq2, sc2 = ct.block_quantize(deq, 32, scale_mode="floor")
+    assert torch.equal(sc2.view(torch.uint8), sc.view(torch.uint8))
+    assert torch.equal(xq2.view(torch.uint8), q)
+
+
+def _native_layout(scales: np.ndarray) -> np.ndarray:
+    """Plain-numpy statement of the native scale layout: dword [I/4][Q][lane][I%4], byte t = scale of row
+    16 I + lane%16, block (4Q + t)*4 + lane/16; padding byte 127."""
+    R, KB = scales.shape
+    R64, KQ = -(-R // 64), -(-KB // 16)
+    out = np.full((R64, KQ, 64, 4, 4), 127, dtype=np.uint8)
+    for row in range(R):
+        for kb in range(KB):
+            I, r = divmod(row, 16)
+            ks, g = divmod(kb, 4)
+            Q, t = divmod(ks, 4)
+            out[I // 4, Q, g * 16 + r, I % 4, t] = scales[row, kb]
+    return out.reshape(-1)
+
+
+@pytest.mark.parametrize("R,K", [(64, 512), (100, 160), (256, 1024), (16, 32)])
+def test_pack_scales_layout(ct, dev, R, K):
+    rng = np.random.default_rng(R + K)
+    s = rng.integers(0, 255, (R, K // 32), dtype=np.uint8)
+    t = torch.from_numpy(s).to(dev)
+    p = ct.pack_scales(t.view(torch.float8_e8m0fnu))
+    want = _native_layout(s)
+    got = p.data.cpu().numpy()[:want.size]
+    assert np.array_equal(got, want)
+    # transposed source (how B_scale is passed) gives the same bytes
+    p2 = ct.pack_scales(t.T.contiguous().view(torch.float8_e8m0fnu), transposed=True)
+    assert torch.equal(p.data, p2.data)
+    if R % 128 == 0 and (K // 32) % 4 == 0:
+        p3 = ct.pack_scales(ct.swizzle_32_4_4(t))
+        assert torch.equal(p.data, p3.data)
+
+
+def test_swizzle_roundtrip_device(ct, dev):
+    # experimental/cuda-lang/test/examples/tk/test_mxfp8_b200_gemm.py:835-837 checks the same round trip
+    s = torch.arange(256 * 8, device=dev, dtype=torch.int32).reshape(256, 8)
+    sw = ct.swizzle_32_4_4(s)
+    assert np.array_equal(sw.cpu().numpy(), O.swizzle_32_4_4(s.cpu().numpy()))
+    assert torch.equal(ct.unswizzle_32_4_4(sw), s)
