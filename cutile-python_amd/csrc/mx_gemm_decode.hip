@@ -6,9 +6,10 @@
 //     of 128 elements) of every tile, so the 8 waves together read each tile's rows contiguously;
 //   * each wave keeps its K-slice of X resident in VGPRs for the whole kernel (X is tiny and shared
 //     by all workgroups through L2), so W is the only stream;
-//   * W fragments go global -> VGPR directly in MFMA operand layout (lane (r, g) holds row r, 32-element
-//     block g of a K-step: the four lane groups read 64 contiguous bytes of a row), the next tile's
-//     loads are issued before the current tile's MFMAs;
+//   * W fragments go global -> VGPR directly in MFMA operand layout (4-bit: lane (r, g) holds row r and
+//     the 32-element block g of a K-step, so the four lane groups read 64 contiguous bytes of a row;
+//     8-bit X: bytes 16 g .. and 64 + 16 g .. of the K-step), the next tile's loads are issued before
+//     the current tile's MFMAs;
 //   * v_mfma_scale_f32_16x16x128_f8f6f4 with mixed formats (W as FP4 first matrix, X as FP8 second
 //     matrix), E8M0 scales read in place from the [N, K/32] / [M, K/32] tensors;
 //   * the 8 K-slice partial sums meet in LDS and 128 threads write the bf16/fp32 result.
@@ -42,8 +43,9 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
       v8i f = {0, 0, 0, 0, 0, 0, 0, 0};
       int sc = 127;
       if (mok && s0 + s < ksteps) {
-        const uint8_t* p = d.X + (int64_t)m * d.ldx + (int64_t)(s0 + s) * 128 + gq * 32;
-        const v4i lo = *(const v4i*)p, hi = *(const v4i*)(p + 16);
+        // 8-bit operand layout of the MFMA: bytes 16 g .. 16 g + 15 and 64 + 16 g .. of the K-step
+        const uint8_t* p = d.X + (int64_t)m * d.ldx + (int64_t)(s0 + s) * 128 + gq * 16;
+        const v4i lo = *(const v4i*)p, hi = *(const v4i*)(p + 64);
         f = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
         sc = d.Xs[(int64_t)m * d.ldxs + (s0 + s) * 4 + gq];
       }

@@ -16,10 +16,15 @@
 // as the second, so a lane ends up with four CONSECUTIVE columns n of one row m and the epilogue can
 // store 8 or 16 contiguous bytes per lane.
 //
-// K-order freedom: lane (r, g) of a 16x16x128 MFMA holds row r and the 32-element block g of the
-// K-step; its scale register byte scales exactly those 32 elements.  A and B use the same block in
-// the same lane group, so the result does not depend on which physical K positions the hardware
-// names a lane's bytes.
+// Operand layout of v_mfma_scale_f32_16x16x128_f8f6f4 (measured on MI355X with one-hot operands):
+//   4-bit formats: lane (r, g) holds row r, K = 32 g + n for nibble n = 0..31 (16 bytes, low nibble
+//                  first): exactly the 32-element scale block g.
+//   8-bit formats: lane (r, g) holds row r, K = 16 g + b in VGPRs 0-3 (bytes b = 0..15) and
+//                  K = 64 + 16 g + b in VGPRs 4-7: two 16-byte pieces, 64 bytes apart in the row.
+//   scales:        the scale of block kb (K = 32 kb .. 32 kb + 31) of row r is read from lane
+//                  (r, kb), byte op_sel of the scale VGPR, for both formats.  For 8-bit data that is
+//                  in general NOT the lane that holds the data.
+//   result:        lane (c, g) holds D[4 g + e][c], e = 0..3 (row index = first matrix's row).
 #include "mx_common.h"
 
 namespace mx {
@@ -62,14 +67,14 @@ __device__ inline int swz(int row) {
   return (row / (16 / CPR)) % CPR;
 }
 
-// Fragment of one 16-row tile for MFMA K-step kk of the stage: 32 K elements of row `row`,
-// block gq.  8-bit formats: 32 bytes (two chunks); 4-bit: 16 bytes in the low four dwords.
+// Fragment of one 16-row tile for MFMA K-step kk of the stage, lane group gq, in the operand layout
+// described at the top of the file.  8-bit formats: two 16-byte chunks; 4-bit: one, in the low dwords.
 template <int RB, int EB>
 __device__ inline v8i load_frag(lds_u8* tile, int row, int kk, int gq, int sw) {
   if constexpr (EB == 8) {
-    const int c = kk * 8 + 2 * gq;
+    const int c = kk * 8 + gq;   // bytes 16 g .. 16 g + 15 and 64 + 16 g .. of the 128-byte K-step
     const v4i lo = *(lds_v4i*)(tile + row * RB + ((c ^ sw) << 4));
-    const v4i hi = *(lds_v4i*)(tile + row * RB + (((c + 1) ^ sw) << 4));
+    const v4i hi = *(lds_v4i*)(tile + row * RB + (((c + 4) ^ sw) << 4));
     return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   } else {
     const int c = kk * 4 + gq;
@@ -218,15 +223,28 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
 
   // ---- scales: one 16-byte load per lane covers 4 row tiles x 4 K-steps ------------------------------
   constexpr int AQ = C::MT / 4, BQ = C::NTL / 4;
-  const v4i* const as_ptr = (const v4i*)g.As + ((int64_t)((m0 + wm0) / 64) * KQ) * 64 + lane;
-  const v4i* const bs_ptr = (const v4i*)(g.Bs + (GROUPED ? (int64_t)expert * g.bs_expert_stride : 0)) +
-                            ((int64_t)((n0 + wn0) / 64) * KQ) * 64 + lane;
+  // the packed tensors hold ceil(rows / 64) row groups; a tile that hangs over the matrix edge re-reads
+  // the last group (its rows are never stored)
+  const v4i* const as_ptr = (const v4i*)g.As + lane;
+  const v4i* const bs_ptr = (const v4i*)(g.Bs + (GROUPED ? (int64_t)expert * g.bs_expert_stride : 0)) + lane;
+  const int a_groups = (g.M + 63) / 64, b_groups = (g.N + 63) / 64;
+  int a_grp[AQ], b_grp[BQ];
+#pragma unroll
+  for (int u = 0; u < AQ; ++u) {
+    const int grp = (m0 + wm0) / 64 + u;
+    a_grp[u] = grp < a_groups ? grp : a_groups - 1;
+  }
+#pragma unroll
+  for (int u = 0; u < BQ; ++u) {
+    const int grp = (n0 + wn0) / 64 + u;
+    b_grp[u] = grp < b_groups ? grp : b_groups - 1;
+  }
   v4i sa[AQ], sb[BQ];
   auto load_scales = [&](int Q) {
 #pragma unroll
-    for (int u = 0; u < AQ; ++u) sa[u] = as_ptr[((int64_t)u * KQ + Q) * 64];
+    for (int u = 0; u < AQ; ++u) sa[u] = as_ptr[((int64_t)a_grp[u] * KQ + Q) * 64];
 #pragma unroll
-    for (int u = 0; u < BQ; ++u) sb[u] = bs_ptr[((int64_t)u * KQ + Q) * 64];
+    for (int u = 0; u < BQ; ++u) sb[u] = bs_ptr[((int64_t)b_grp[u] * KQ + Q) * 64];
   };
 
   v4f acc[C::MT][C::NTL];
