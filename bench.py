@@ -1,0 +1,320 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-scaled (MX) matmul path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2|c3|c4|c5] [--no-cpu]
+
+A "step" is one call of the hot path -- block_scaled_matmul(A, A_scale, B, B_scale, out_dtype=bf16) with
+the reference's tensor layouts (plain (M, K/32) / (K/32, N) E8M0 scales, so the per-call scale re-layout
+is inside the step) -- on synthetic operands already resident in HBM.  The headline workload is the
+configuration the metric is quoted on: MXFP8 E4M3 x E4M3, M = N = K = 8192, bf16 output.  The other
+single-GPU configurations of the metric (MXFP4 8192^3, the M = 32 decode GEMM, the MoE grouped GEMM) are
+timed the same way and reported under "extra".
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel of the headline workload: algorithmic
+flops per launch divided by the kernel's average duration, measured with HIP events on the launch stream
+around launches of the GEMM kernel alone (scales pre-packed, so no other kernel runs in that region).
+`cpu_baseline` times the oracle's dequantize + fp32 matmul on this host's cores on an N-slice of the same
+workload.  Operand sets are rotated so that no launch finds its inputs in L2 / Infinity Cache.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import pathlib
+import sys
+import time
+
+ROOT = pathlib.Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT / "cutile-python_amd"))
+sys.path.insert(0, str(ROOT))
+
+import numpy as np  # noqa: E402
+import torch  # noqa: E402
+
+PEAK_TFLOPS = {"mxfp8": 5033.0, "mxfp4": 10066.0}   # MI355X dense MFMA peaks (vendor figures)
+PEAK_HBM_GBS = 8000.0
+METRIC = "MX GEMM TFLOP/s (+% MFMA peak) 8192^3 MXFP8/MXFP4; GB/s at M=32 decode"
+
+
+def _sync():
+    torch.cuda.synchronize()
+
+
+def _time_wall(fn, steps, warmup):
+    """Contract timing: W untimed warm-up steps, then exactly K steps between synchronisations."""
+    for i in range(warmup):
+        fn(i)
+    _sync()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(warmup + i)
+    _sync()
+    return (time.perf_counter() - t0) / steps
+
+
+def _time_events(fn, steps, warmup):
+    """Average duration of one launch from HIP events recorded on the launch stream."""
+    for i in range(warmup):
+        fn(i)
+    _sync()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        fn(warmup + i)
+    stop.record()
+    _sync()
+    return start.elapsed_time(stop) * 1e-3 / steps
+
+
+def _quantized(ct, rows, K, fmt, seed, dev, dist, std=1.0, cpu_seeded=True):
+    """(storage, scale) on the device.  The first operand set of every workload comes from a seeded CPU
+    generator (the workload definition); rotation copies are drawn on the device."""
+    if cpu_seeded:
+        g = torch.Generator().manual_seed(seed)
+        x = torch.randn((rows, K), generator=g) if dist == "randn" else torch.rand((rows, K), generator=g) * 12 - 6
+        x = (x * std).to(dev)
+    else:
+        g = torch.Generator(device=dev).manual_seed(seed)
+        x = torch.randn((rows, K), generator=g, device=dev) if dist == "randn" else \
+            torch.rand((rows, K), generator=g, device=dev) * 12 - 6
+        x = x * std
+    q, s = ct.block_quantize(x, 32, fmt, scale_mode="floor")
+    del x
+    return q, s
+
+
+def _oracle_rows(O, a_q, a_s, b_q, b_s, rows, a_fmt, b_fmt):
+    """CPU oracle of C[rows, :] for K-contiguous operands a (M, K) and b (N, K)."""
+    def codes(t, fmt):
+        u = t.view(torch.uint8).cpu().numpy()
+        return O.unpack_fp4(u) if fmt == O.E2M1 else u
+    a = O.dequantize(codes(a_q[rows], a_fmt), a_s[rows].view(torch.uint8).cpu().numpy(), a_fmt)
+    b = O.dequantize(codes(b_q, b_fmt), b_s.view(torch.uint8).cpu().numpy(), b_fmt)
+    return a @ b.T
+
+
+def _check_rows(O, c, ref, rows, tol, what):
+    err = O.rel_fro(c[rows].float().cpu(), ref)
+    if not err <= tol:
+        raise SystemExit(f"bench: {what}: relative Frobenius error {err:.3e} exceeds {tol}")
+    return err
+
+
+def bench_gemm(ct, O, dev, M, N, K, fmt, dist, steps, warmup, check, nsets=3):
+    """Square / large GEMM configurations (MXFP8 or MXFP4, bf16 out)."""
+    tfmt = torch.float8_e4m3fn if fmt == O.E4M3 else "e2m1"
+    kw = {} if fmt == O.E4M3 else {"a_format": "e2m1", "b_format": "e2m1"}
+    sets = []
+    for i in range(nsets):
+        a_q, a_s = _quantized(ct, M, K, tfmt, 1234 + 2 * i, dev, dist, cpu_seeded=(i == 0))
+        b_q, b_s = _quantized(ct, N, K, tfmt, 1235 + 2 * i, dev, dist, cpu_seeded=(i == 0))
+        sets.append((a_q, a_s, b_q, b_s, torch.empty((M, N), dtype=torch.bfloat16, device=dev)))
+    err = None
+    if check:
+        a_q, a_s, b_q, b_s, c = sets[0]
+        ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, C=c, **kw)
+        rows = torch.arange(0, M, max(1, M // 32))[:32]
+        err = _check_rows(O, c, _oracle_rows(O, a_q, a_s, b_q, b_s, rows, fmt, fmt), rows, 8e-3, f"{fmt} {M}x{N}x{K}")
+
+    def step(i):
+        a_q, a_s, b_q, b_s, c = sets[i % nsets]
+        ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, C=c, **kw)
+
+    t_step = _time_wall(step, steps, warmup)
+    packed = [(ct.pack_scales(s[1]), ct.pack_scales(s[3])) for s in sets]
+
+    def kernel_only(i):
+        a_q, _, b_q, _, c = sets[i % nsets]
+        pa, pb = packed[i % nsets]
+        ct.block_scaled_matmul(a_q, pa, b_q.T, pb, C=c, **kw)
+
+    t_kernel = _time_events(kernel_only, steps, warmup)
+    flops = 2.0 * M * N * K
+    return {"ms_per_step": t_step * 1e3, "tflops": flops / t_step * 1e-12, "kernel_ms": t_kernel * 1e3,
+            "kernel_tflops": flops / t_kernel * 1e-12, "rel_fro_vs_oracle": err, "flops": flops, "sets": sets}
+
+
+def bench_decode(ct, O, dev, steps, warmup, check, nsets=8):
+    """Decode-shaped mixed GEMM: X MXFP8 (32, 8192) x W MXFP4 (28672, 8192)^T, bf16 out.  HBM bound; the
+    121 MiB working set fits in the Infinity Cache, so 8 weight sets are rotated."""
+    M, N, K = 32, 28672, 8192
+    x_q, x_s = _quantized(ct, M, K, torch.float8_e4m3fn, 2001, dev, "randn")
+    ws = []
+    for i in range(nsets):
+        w_q, w_s = _quantized(ct, N, K, "e2m1", 2002 + i, dev, "randn", std=0.02, cpu_seeded=(i == 0))
+        ws.append((w_q, w_s, torch.empty((M, N), dtype=torch.bfloat16, device=dev)))
+    err = None
+    if check:
+        w_q, w_s, c = ws[0]
+        ct.block_scaled_matmul(x_q, x_s, w_q.T, w_s.T, b_format="e2m1", C=c)
+        ref = _oracle_rows(O, x_q, x_s, w_q, w_s, torch.arange(M), O.E4M3, O.E2M1)
+        err = _check_rows(O, c, ref, torch.arange(M), 8e-3, "decode 32x28672x8192")
+
+    def step(i):
+        w_q, w_s, c = ws[i % nsets]
+        ct.block_scaled_matmul(x_q, x_s, w_q.T, w_s.T, b_format="e2m1", C=c)
+
+    t_wall = _time_wall(step, steps, warmup)
+    # The kernel runs ~20 us, less than the host needs to issue a launch from Python, so the kernel's own
+    # duration is taken from a captured graph of one launch per weight set, replayed between HIP events.
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(nsets):
+            step(i)
+    reps = max(1, (steps + nsets - 1) // nsets)
+    t = _time_events(lambda i: graph.replay(), reps, 2) / nsets
+    nbytes = M * K + M * K // 32 + N * K // 2 + N * K // 32 + M * N * 2     # 126 885 888
+    return {"ms_per_step": t_wall * 1e3, "kernel_ms": t * 1e3, "gbs": nbytes / t * 1e-9,
+            "gbs_wall": nbytes / t_wall * 1e-9, "bytes": nbytes, "rel_fro_vs_oracle": err}
+
+
+def bench_moe(ct, O, dev, steps, warmup, check):
+    """MoE grouped MXFP8 GEMM: 4096 tokens, hidden 4096, 8 experts x 14336, top-2 (8192 routed rows)."""
+    T, K, N, E, topk, tile = 4096, 4096, 14336, 8, 2, 256
+    x_q, x_s = _quantized(ct, T, K, torch.float8_e4m3fn, 3001, dev, "randn")
+    w_q, w_s = _quantized(ct, E * N, K, torch.float8_e4m3fn, 3002, dev, "randn", std=0.02, cpu_seeded=False)
+    W, Ws = w_q.view(E, N, K), w_s.view(E, N, K // 32)
+    g = torch.Generator().manual_seed(3003)
+    ids = torch.topk(torch.rand((T, E), generator=g), topk, dim=1).indices.to(dev)
+    sid, eid = ct.moe_align_tile_size(ids, tile, E)
+    C = torch.empty((T, topk, N), dtype=torch.bfloat16, device=dev)
+    err = None
+    if check:
+        ct.invoke_fused_moe_scaled(x_q, x_s, W, Ws, C, None, sid, eid, False, topk, tile)
+        # oracle on the rows of 16 tokens, one weight dequantisation per expert
+        toks = torch.arange(0, T, T // 16)[:16]
+        a = O.dequantize(x_q[toks].view(torch.uint8).cpu().numpy(), x_s[toks].view(torch.uint8).cpu().numpy(), O.E4M3)
+        ids_cpu = ids.cpu()
+        num = den = 0.0
+        for e in sorted(set(ids_cpu[toks].reshape(-1).tolist())):
+            w = O.dequantize(W[e].view(torch.uint8).cpu().numpy(), Ws[e].view(torch.uint8).cpu().numpy(), O.E4M3)
+            for ti, t in enumerate(toks.tolist()):
+                for j in range(topk):
+                    if int(ids_cpu[t, j]) != e:
+                        continue
+                    ref = a[ti] @ w.T
+                    got = C[t, j].float().cpu()
+                    num += float(((got - ref).double() ** 2).sum())
+                    den += float((ref.double() ** 2).sum())
+        err = (num / den) ** 0.5
+        if not err <= 8e-3:
+            raise SystemExit(f"bench: MoE grouped GEMM: relative Frobenius error {err:.3e} exceeds 8e-3")
+
+    def step(i):
+        ct.invoke_fused_moe_scaled(x_q, x_s, W, Ws, C, None, sid, eid, False, topk, tile)
+
+    t_step = _time_wall(step, steps, warmup)
+    pW = ct.pack_scales(Ws)
+
+    def kernel_mostly(i):
+        ct.invoke_fused_moe_scaled(x_q, x_s, W, pW, C, None, sid, eid, False, topk, tile)
+
+    t_k = _time_events(kernel_mostly, steps, warmup)
+    flops = 2.0 * T * topk * K * N
+    return {"ms_per_step": t_step * 1e3, "tflops": flops / t_step * 1e-12, "kernel_ms": t_k * 1e3,
+            "kernel_tflops": flops / t_k * 1e-12, "rel_fro_vs_oracle": err, "padded_rows": int(sid.numel())}
+
+
+def cpu_baseline_c2(O, sets, budget_s=12.0):
+    """The reference's check (dequantize to fp32, torch matmul; samples/BlockScaledMatMul.py:358-364) timed on
+    the host cores on an N-slice of the headline workload, sized from a probe to about `budget_s`."""
+    a_q, a_s, b_q, b_s, _ = sets[0]
+    M, K = a_q.shape
+    a_c, a_sc = a_q.view(torch.uint8).cpu().numpy(), a_s.view(torch.uint8).cpu().numpy()
+    cores = os.cpu_count() or 1
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        pass
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+
+    def run(n):
+        b_c, b_sc = b_q[:n].view(torch.uint8).cpu().numpy(), b_s[:n].view(torch.uint8).cpu().numpy()
+        t0 = time.perf_counter()
+        a = O.dequantize(a_c, a_sc, O.E4M3)
+        b = O.dequantize(b_c, b_sc, O.E4M3)
+        c = a @ b.T
+        dt = time.perf_counter() - t0
+        return dt, float(c[0, 0])
+
+    t_probe, _ = run(64)
+    n = int(min(8192, max(64, 64 * budget_s / max(t_probe, 1e-3) // 64 * 64)))
+    dt, _ = run(n)
+    tflops = 2.0 * M * n * K / dt * 1e-12
+    return {"value": tflops, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"torch dequantize + fp32 matmul of the 8192 x {n} x 8192 column slice of the workload, "
+                      f"{dt:.1f} s wall, one run"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c5 (default: all)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-check", action="store_true", help="skip the correctness check before timing")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU (the path has no cross-GPU exchange: weights "
+                         "would be sharded along N, see DESIGN.md); run with --gpus 1")
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py: no GPU visible")
+    import cutile_amd as ct
+    from oracle import mx_oracle as O   # checker + cpu_baseline leg only
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if ct.lib().mx_device_check() != 0:
+        raise SystemExit("bench.py: " + ct._lib.last_error())
+    want = set(filter(None, a.only.split(","))) or {"c2", "c3", "c4", "c5"}
+    check = not a.no_check
+    extra = {}
+    if "c4" in want:
+        r = bench_gemm(ct, O, dev, 8192, 8192, 8192, O.E2M1, "uniform6", a.steps, a.warmup, check)
+        r.pop("sets")
+        extra["c4_mxfp4_8192"] = {"tflops": r["tflops"], "ms_per_step": r["ms_per_step"],
+                                  "kernel_tflops": r["kernel_tflops"], "frac_of_mxfp4_peak": r["kernel_tflops"] / PEAK_TFLOPS["mxfp4"],
+                                  "rel_fro_vs_oracle": r["rel_fro_vs_oracle"]}
+        torch.cuda.empty_cache()
+    if "c3" in want:
+        r = bench_decode(ct, O, dev, max(a.steps, 50), a.warmup, check)
+        extra["c3_decode_m32"] = {"gbs": r["gbs"], "kernel_us": r["kernel_ms"] * 1e3, "gbs_wall_clock": r["gbs_wall"],
+                                  "frac_of_hbm_peak": r["gbs"] / PEAK_HBM_GBS, "bytes": r["bytes"],
+                                  "rel_fro_vs_oracle": r["rel_fro_vs_oracle"]}
+        torch.cuda.empty_cache()
+    if "c5" in want:
+        r = bench_moe(ct, O, dev, a.steps, a.warmup, check)
+        extra["c5_moe_grouped_mxfp8"] = {"tflops": r["tflops"], "ms_per_step": r["ms_per_step"],
+                                         "kernel_tflops": r["kernel_tflops"],
+                                         "frac_of_mxfp8_peak": r["kernel_tflops"] / PEAK_TFLOPS["mxfp8"],
+                                         "padded_rows": r["padded_rows"], "rel_fro_vs_oracle": r["rel_fro_vs_oracle"]}
+        torch.cuda.empty_cache()
+    out = {"metric": METRIC, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "mxfp8_e4m3 (e8m0 scales, fp32 accumulate, bf16 out)",
+           "data": "synthetic", "extra": extra}
+    if "c2" in want:
+        r = bench_gemm(ct, O, dev, 8192, 8192, 8192, O.E4M3, "randn", a.steps, a.warmup, check)
+        out.update({
+            "value": r["tflops"], "ms_per_step": r["ms_per_step"],
+            "config": {"workload": "MXFP8 E4M3 x E4M3 block-scaled GEMM, M=N=K=8192, E8M0 scale per 32 along K "
+                                   "(floor rule), A row-major MxK, B column-major KxN, fp32 accumulate, bf16 output; "
+                                   "one step = one block_scaled_matmul call incl. scale re-layout",
+                       "M": 8192, "N": 8192, "K": 8192, "operand_sets_rotated": 3},
+            "rel_fro_vs_oracle": r["rel_fro_vs_oracle"],
+            "roofline": {"bound": "mfma", "achieved": r["kernel_tflops"], "peak": PEAK_TFLOPS["mxfp8"],
+                         "unit": "TFLOP/s", "frac": r["kernel_tflops"] / PEAK_TFLOPS["mxfp8"], "traffic": None,
+                         "kernel": "gemm_kernel<Cfg<e4m3,e4m3,256,256,2,4>,bf16>", "kernel_ms": r["kernel_ms"],
+                         "flops_per_launch": r["flops"]},
+        })
+        if not a.no_cpu:
+            out["cpu_baseline"] = cpu_baseline_c2(O, r["sets"])
+    else:
+        out.update({"value": None, "ms_per_step": None, "config": {"workload": "partial run: " + ",".join(sorted(want))}})
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -143,6 +143,22 @@ def _scale_desc(s, rows: int, K: int, block: int, is_b: bool):
     return L.desc(_as_u8(s), code), L.MX_SCALE_2D
 
 
+_WS_CACHE: dict = {}
+
+
+def _workspace(dev: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+    """Scratch for the per-call scale re-layout: one buffer per (device, stream), grown on demand, so the
+    hot path does not go through the allocator.  Kernels that use it are ordered on that stream."""
+    if nbytes <= 0:
+        return None
+    key = (dev.index, L.stream_ptr(dev))
+    buf = _WS_CACHE.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        _WS_CACHE[key] = buf
+    return buf
+
+
 def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kernel, block):
     dev = A.device
     and_, bnd = A.dim(), B.dim()
@@ -157,13 +173,11 @@ def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kerne
     o = _opts(accumulate, la, lb, kernel, block)
     lib = L.lib()
     need = lib.mx_gemm_workspace_bytes(M, N, K, ctypes.byref(o))
-    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev) if need else None
+    ws = _workspace(dev, need)
     with torch.cuda.device(dev):
         rc = lib.mx_gemm(ctypes.byref(dA), ctypes.byref(dAs), ctypes.byref(dB), ctypes.byref(dBs),
                          ctypes.byref(dC), ctypes.byref(o), ws.data_ptr() if ws is not None else None,
                          need, L.stream_ptr(dev))
-    if ws is not None:
-        ws.record_stream(torch.cuda.current_stream(dev))
     _check(rc)
     return C
 
@@ -492,11 +506,10 @@ def invoke_fused_moe_scaled(A: torch.Tensor, A_scale: torch.Tensor, B: torch.Ten
     eids = sorted_expert_ids.to(torch.int32).contiguous()
     lib = L.lib()
     need = lib.mx_gemm_grouped_workspace_bytes(ids.numel(), N, K, E, ctypes.byref(o))
-    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    ws = _workspace(dev, max(need, 1))
     with torch.cuda.device(dev):
         rc = lib.mx_gemm_grouped(ctypes.byref(dA), ctypes.byref(dAs), ctypes.byref(dB), ctypes.byref(dBs),
                                  ctypes.byref(dC), w.data_ptr() if w is not None else None, ids.data_ptr(),
                                  ids.numel(), eids.data_ptr(), tile_m, num_token_replicas, num_valid,
                                  ctypes.byref(o), ws.data_ptr(), need, L.stream_ptr(dev))
-    ws.record_stream(torch.cuda.current_stream(dev))
     _check(rc)
