@@ -257,6 +257,9 @@ def main():
     ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c5 (default: all)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the correctness check before timing")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy kernel (a known-size reference for "
+                         "scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (the path has no cross-GPU exchange: weights "
@@ -269,6 +272,12 @@ def main():
     torch.cuda.set_device(dev)
     if ct.lib().mx_device_check() != 0:
         raise SystemExit("bench.py: " + ct._lib.last_error())
+    if a.calib_copy:
+        src = torch.empty(64 << 20, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)          # 256 MiB read + 256 MiB written by one elementwise copy kernel
+        _sync()
+        del src, dst
     want = set(filter(None, a.only.split(","))) or {"c2", "c3", "c4", "c5"}
     check = not a.no_check
     extra = {}

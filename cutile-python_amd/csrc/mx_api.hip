@@ -218,7 +218,8 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
     if (why) kernel = MX_KERNEL_GENERIC;
     else if (M <= 32 && A->dtype != MX_E2M1 && B->dtype == MX_E2M1 && o.a_scale_layout == MX_SCALE_2D &&
              o.b_scale_layout == MX_SCALE_2D && Bs->stride[0] == 1 && As->stride[1] == 1 && K % 512 == 0 &&
-             K <= 8192 && N % 16 == 0 && Bs->stride[1] % 16 == 0 && ((uintptr_t)Bs->ptr) % 16 == 0)
+             K <= 8192 && N % 16 == 0 && Bs->stride[1] % 16 == 0 && ((uintptr_t)Bs->ptr) % 16 == 0 &&
+             N * b_ld < ((int64_t)1 << 31) && As->stride[0] % 16 == 0 && ((uintptr_t)As->ptr) % 16 == 0)
       kernel = MX_KERNEL_DECODE;
     else if (M > 128 && N > 128 && (int64_t)M * N >= (int64_t)1024 * 1024) kernel = MX_KERNEL_MFMA_256x256;
     else kernel = MX_KERNEL_MFMA_128x128;
@@ -270,8 +271,8 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
       return set_error(MX_ERR_LAYOUT, "the decode kernel reads K-contiguous 2-D scales in place");
     if (A->dtype == MX_E2M1 || B->dtype != MX_E2M1)
       return set_error(MX_ERR_DTYPE, "the decode kernel takes 8-bit activations and FP4 weights");
-    if (K % 512 != 0 || N % 16 != 0)
-      return set_error(MX_ERR_SHAPE, "the decode kernel needs K %% 512 == 0 and N %% 16 == 0");
+    if (K % 512 != 0 || K > 8192 || N % 16 != 0)
+      return set_error(MX_ERR_SHAPE, "the decode kernel needs K %% 512 == 0, K <= 8192 and N %% 16 == 0");
     DecodeArgs d = {};
     d.X = (const uint8_t*)A->ptr; d.Xs = (const uint8_t*)As->ptr;
     d.W = (const uint8_t*)B->ptr; d.Ws = (const uint8_t*)Bs->ptr; d.C = C->ptr;

@@ -94,6 +94,7 @@ struct GemmArgs {
   int64_t b_expert_stride;   // bytes between experts in B
   int64_t bs_expert_stride;  // dwords between experts in Bs
   int64_t a_rows;            // rows of the A tensor (for the buffer descriptor)
+  int32_t stagger;           // 1: workgroups start their K walk at different quads
 };
 
 int launch_gemm_mfma(const GemmArgs& g, int kernel_id, hipStream_t stream);

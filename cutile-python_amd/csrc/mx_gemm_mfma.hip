@@ -25,6 +25,8 @@
 //                  (r, kb), byte op_sel of the scale VGPR, for both formats.  For 8-bit data that is
 //                  in general NOT the lane that holds the data.
 //   result:        lane (c, g) holds D[4 g + e][c], e = 0..3 (row index = first matrix's row).
+#include <stdlib.h>
+
 #include "mx_common.h"
 
 namespace mx {
@@ -128,7 +130,7 @@ __device__ inline void store4<uint16_t>(uint16_t* p, const v4f& v, bool accumula
   }
 }
 
-template <class C, typename OutT, bool GROUPED>
+template <class C, typename OutT, bool GROUPED, int PIPE>
 __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
   lds_u8* const smem = (lds_u8*)smem_generic;
@@ -141,7 +143,7 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
 
   // ---- tile of C owned by this workgroup: XCD-aware, then grouped along M --------------------------
   const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
-  int tile_m, tile_n;
+  int tile_m, tile_n, tile_lid;
   {
     const int total = tiles_m * tiles_n;
     const int pid = blockIdx.x;
@@ -156,6 +158,7 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
     const int in = lid % in_group;
     tile_m = first_m + in % gsz;
     tile_n = in / gsz;
+    tile_lid = lid;
   }
   const int m0 = tile_m * C::BM, n0 = tile_n * C::BN;
 
@@ -182,6 +185,7 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
     const int col = (pos ^ swz<C::A_CPR>(row)) * 16;
     a_col[q] = col;
     int64_t grow = m0 + row;
+    if constexpr (PIPE == 6) grow = row & 15;          // timing experiment: every load hits in cache
     bool ok = grow < g.M;
     if constexpr (GROUPED) {
       const int id = ok ? g.sorted_token_ids[grow] : 0x7FFFFFFF;
@@ -196,27 +200,28 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
     const int row = slot / C::B_CPR, pos = slot % C::B_CPR;
     const int col = (pos ^ swz<C::B_CPR>(row)) * 16;
     b_col[q] = col;
-    const int64_t grow = n0 + row;
+    int64_t grow = n0 + row;
+    if constexpr (PIPE == 6) grow = row & 15;
     b_voff[q] = grow < g.N ? (uint32_t)(grow * g.ldb + col) : kOobOffset;
   }
 
-  auto issue_stage = [&](int s, int buf) {
+  // One 16-byte-per-lane LDS-DMA load of stage s: idx < A_LOADS moves A rows, the rest B rows.  `live`
+  // false (no such stage) turns the load into a zero fill of the idle buffer, which keeps the
+  // instruction stream branch-free.
+  constexpr int TOTAL_LOADS = C::A_LOADS + C::B_LOADS;
+  auto issue_one = [&](int idx, int s, int buf, bool live) {
     lds_u8* const abase = smem + buf * C::STAGE;
-    lds_u8* const bbase = abase + C::A_STAGE;
-    const int ka = s * C::A_RB, kb = s * C::B_RB;
-    const bool tail_a = ka + C::A_RB > Kb_a, tail_b = kb + C::B_RB > Kb_b;   // uniform
-#pragma unroll
-    for (int q = 0; q < C::A_LOADS; ++q) {
+    if (idx < C::A_LOADS) {
+      const int q = idx, ka = s * C::A_RB;
       uint32_t v = a_voff[q];
-      if (tail_a && ka + a_col[q] >= Kb_a) v = kOobOffset;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_void*)(abase + (q * C::NW + wave) * 1024),
-                                               16, v, ka, 0, 0);
-    }
-#pragma unroll
-    for (int q = 0; q < C::B_LOADS; ++q) {
+      if (!live || ka + a_col[q] >= Kb_a) v = kOobOffset;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_void*)(abase + (q * C::NW + wave) * 1024), 16, v,
+                                               ka, 0, 0);
+    } else {
+      const int q = idx - C::A_LOADS, kb = s * C::B_RB;
       uint32_t v = b_voff[q];
-      if (tail_b && kb + b_col[q] >= Kb_b) v = kOobOffset;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(bbase + (q * C::NW + wave) * 1024),
+      if (!live || kb + b_col[q] >= Kb_b) v = kOobOffset;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(abase + C::A_STAGE + (q * C::NW + wave) * 1024),
                                                16, v, kb, 0, 0);
     }
   };
@@ -239,12 +244,14 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
     const int grp = (n0 + wn0) / 64 + u;
     b_grp[u] = grp < b_groups ? grp : b_groups - 1;
   }
-  v4i sa[AQ], sb[BQ];
-  auto load_scales = [&](int Q) {
+  // scales of the current K-quad and, prefetched one quad ahead, of the next
+  v4i sa[AQ], sb[BQ], sa_n[AQ], sb_n[BQ];
+  auto load_scales = [&](int Q, v4i* da, v4i* db) {
+    const int Qc = Q < KQ ? Q : KQ - 1;
 #pragma unroll
-    for (int u = 0; u < AQ; ++u) sa[u] = as_ptr[((int64_t)a_grp[u] * KQ + Q) * 64];
+    for (int u = 0; u < AQ; ++u) da[u] = as_ptr[((int64_t)a_grp[u] * KQ + Qc) * 64];
 #pragma unroll
-    for (int u = 0; u < BQ; ++u) sb[u] = bs_ptr[((int64_t)b_grp[u] * KQ + Q) * 64];
+    for (int u = 0; u < BQ; ++u) db[u] = bs_ptr[((int64_t)b_grp[u] * KQ + Qc) * 64];
   };
 
   v4f acc[C::MT][C::NTL];
@@ -254,29 +261,52 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
     for (int j = 0; j < C::NTL; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
   const int swa = swz<C::A_CPR>(r), swb = swz<C::B_CPR>(r);
+  // DMA loads of the next stage are spread over the first half of the MFMA tiles of the current one
+  constexpr int LOAD_ITERS = C::MT >= 2 ? C::MT / 2 : 1;
+  constexpr int LPI = (TOTAL_LOADS + LOAD_ITERS - 1) / LOAD_ITERS;
 
-  issue_stage(0, 0);
+  // K is walked in quads of four 128-element steps.  Workgroups that run side by side start at different
+  // quads (and wrap around): with power-of-two row pitches all rows of a stage live in the same memory
+  // channel, and without the stagger every workgroup would ask that one channel at the same time.
+  constexpr int SPQ = 4 / C::KSUB;   // stages per quad
+  const int q_start = (g.stagger && ksteps % 4 == 0) ? tile_lid % KQ : 0;
+  load_scales(q_start, sa, sb);
+#pragma unroll
+  for (int idx = 0; idx < TOTAL_LOADS; ++idx) issue_one(idx, q_start * SPQ, 0, true);
   int buf = 0;
-  for (int Q = 0; Q < KQ; ++Q) {
-    load_scales(Q);
+  for (int Qi = 0; Qi < KQ; ++Qi) {
+    const int Q = Qi + q_start < KQ ? Qi + q_start : Qi + q_start - KQ;
+    const int Qn = Q + 1 < KQ ? Q + 1 : 0;
+    load_scales(Qn, sa_n, sb_n);
 #pragma unroll
     for (int t0 = 0; t0 < 4; t0 += C::KSUB) {
-      const int s = Q * (4 / C::KSUB) + t0 / C::KSUB;
-      if (s < nstages) {
+      const int s = Q * SPQ + t0 / C::KSUB;
+      const int it = Qi * SPQ + t0 / C::KSUB;        // position in the (rotated) walk
+      if (it < nstages) {
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this thread's LDS-DMA of stage s landed
-        __syncthreads();                      // everyone's landed; everyone left stage s-1's buffer
-        if (s + 1 < nstages) issue_stage(s + 1, buf ^ 1);
+        if constexpr (PIPE != 4 && PIPE != 5)
+          __syncthreads();                    // everyone's landed; everyone left stage s-1's buffer
+        const bool more = it + 1 < nstages;
+        const int sn = (t0 / C::KSUB + 1 < SPQ) ? s + 1 : Qn * SPQ;   // stage that follows in the walk
+        if constexpr (PIPE == 0) {
+#pragma unroll
+          for (int idx = 0; idx < TOTAL_LOADS; ++idx) issue_one(idx, sn, buf ^ 1, more);
+        }
         lds_u8* const atile = smem + buf * C::STAGE + (wm0 + r) * C::A_RB;
         lds_u8* const btile = smem + buf * C::STAGE + C::A_STAGE + (wn0 + r) * C::B_RB;
 #pragma unroll
         for (int kk = 0; kk < C::KSUB; ++kk) {
           v8i bf[C::NTL];
 #pragma unroll
-          for (int j = 0; j < C::NTL; ++j)
-            bf[j] = load_frag<C::B_RB, C::B_EB>(btile, 16 * j, kk, gq, swb);
+          for (int j = 0; j < C::NTL; ++j) {
+            if constexpr (PIPE == 3 || PIPE == 5) bf[j] = (v8i){s, j, kk, gq, swb, lane, 3, 4};
+            else bf[j] = load_frag<C::B_RB, C::B_EB>(btile, 16 * j, kk, gq, swb);
+          }
 #pragma unroll
           for (int i = 0; i < C::MT; ++i) {
-            const v8i af = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
+            v8i af;
+            if constexpr (PIPE == 3 || PIPE == 5) af = (v8i){s, i, kk, gq, swa, lane, 1, 2};
+            else af = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
 #pragma unroll
             for (int j = 0; j < C::NTL; ++j) {
               // compile-time K-step index within the quad selects the scale byte
@@ -289,11 +319,24 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
               else
                 acc[i][j] = mfma_scaled<C::BF, C::AF, 3>(bf[j], af, acc[i][j], sb[j / 4][j % 4], sa[i / 4][i % 4]);
             }
+            if constexpr (PIPE == 1 || PIPE == 3 || PIPE == 6 || PIPE == 7) {
+              if (kk == 0 && i < LOAD_ITERS) {
+#pragma unroll
+                for (int l = 0; l < LPI; ++l)
+                  if (i * LPI + l < (PIPE == 7 ? C::A_LOADS : TOTAL_LOADS)) issue_one(i * LPI + l, sn, buf ^ 1, more);
+              }
+              // keep the DMA loads in the tile iteration they were written in; everything else may move
+              __builtin_amdgcn_sched_barrier(0x78F);
+            }
           }
         }
         buf ^= 1;
       }
     }
+#pragma unroll
+    for (int u = 0; u < AQ; ++u) sa[u] = sa_n[u];
+#pragma unroll
+    for (int u = 0; u < BQ; ++u) sb[u] = sb_n[u];
   }
 
   // ---- epilogue: lane (r, gq) of tile (i, j) holds C[m0+wm0+16i+r][n0+wn0+16j+4gq .. +3] -----------
@@ -324,9 +367,9 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
   }
 }
 
-template <class C, typename OutT, bool GROUPED>
+template <class C, typename OutT, bool GROUPED, int PIPE = 1>
 int launch_one(const GemmArgs& g, hipStream_t stream) {
-  auto kern = gemm_kernel<C, OutT, GROUPED>;
+  auto kern = gemm_kernel<C, OutT, GROUPED, PIPE>;
   static int attr_done = 0;   // benign race: the attribute call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -347,13 +390,30 @@ int launch_one(const GemmArgs& g, hipStream_t stream) {
 template <int BM, int BN, int WGM, int WGN>
 int launch_fmt(const GemmArgs& g, hipStream_t stream) {
   const bool grouped = g.sorted_token_ids != nullptr;
+  // tuning aid: MXGEMM_PIPE=0 selects the variant that issues all DMA loads of a stage in one burst
+  static const int pipe_env = [] { const char* e = getenv("MXGEMM_PIPE"); return e ? atoi(e) : 1; }();
+  static const int stagger_env = [] { const char* e = getenv("MXGEMM_STAGGER"); return e ? atoi(e) : 0; }();
+  GemmArgs gs = g;
+  gs.stagger = stagger_env;
+  if (pipe_env != 1 && g.a_fmt == MX_E4M3 && g.b_fmt == MX_E4M3 && g.c_dtype == MX_BF16 && !grouped) {
+    using C = Cfg<MX_E4M3, MX_E4M3, BM, BN, WGM, WGN>;
+    switch (pipe_env) {
+      case 0: return launch_one<C, uint16_t, false, 0>(gs, stream);
+      case 2: return launch_one<C, uint16_t, false, 2>(gs, stream);   // no DMA in the loop
+      case 3: return launch_one<C, uint16_t, false, 3>(gs, stream);   // no LDS reads
+      case 4: return launch_one<C, uint16_t, false, 4>(gs, stream);   // no DMA, no barrier
+      case 5: return launch_one<C, uint16_t, false, 5>(gs, stream);   // MFMA only
+      case 6: return launch_one<C, uint16_t, false, 6>(gs, stream);   // all loads cache-resident
+      case 7: return launch_one<C, uint16_t, false, 7>(gs, stream);   // only the A loads
+    }
+  }
 #define MX_CASE(AFMT, BFMT)                                                                        \
   if (g.a_fmt == AFMT && g.b_fmt == BFMT) {                                                        \
     using C = Cfg<AFMT, BFMT, BM, BN, WGM, WGN>;                                                   \
     if (g.c_dtype == MX_F32)                                                                       \
-      return grouped ? launch_one<C, float, true>(g, stream) : launch_one<C, float, false>(g, stream); \
-    return grouped ? launch_one<C, uint16_t, true>(g, stream)                                      \
-                   : launch_one<C, uint16_t, false>(g, stream);                                    \
+      return grouped ? launch_one<C, float, true>(gs, stream) : launch_one<C, float, false>(gs, stream); \
+    return grouped ? launch_one<C, uint16_t, true>(gs, stream)                                      \
+                   : launch_one<C, uint16_t, false>(gs, stream);                                    \
   }
   MX_CASE(MX_E4M3, MX_E4M3)
   MX_CASE(MX_E5M2, MX_E5M2)
