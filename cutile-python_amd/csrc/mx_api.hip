@@ -1,6 +1,7 @@
 // C ABI of libmxgemm.so: argument validation and kernel dispatch.  See include/mxgemm.h.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "mx_common.h"
@@ -21,6 +22,13 @@ namespace {
 
 inline bool is_elem(int d) { return d == MX_E4M3 || d == MX_E5M2 || d == MX_E2M1; }
 inline int64_t round256(int64_t b) { return (b + 255) & ~(int64_t)255; }
+
+// kernel MX_KERNEL_AUTO uses for large problems; MXGEMM_PP=0 (read once) selects the non-ping-pong
+// 256x256 kernel instead, for side-by-side timing
+int big_tile_kernel() {
+  static const int pp = [] { const char* e = getenv("MXGEMM_PP"); return e ? atoi(e) : 1; }();
+  return pp ? MX_KERNEL_MFMA_PINGPONG : MX_KERNEL_MFMA_256x256;
+}
 
 const mx_gemm_opts kDefaultOpts = {sizeof(mx_gemm_opts), 0, MX_SCALE_2D, MX_SCALE_2D, MX_KERNEL_AUTO, 32, {0, 0}};
 
@@ -221,7 +229,7 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
              K <= 8192 && N % 16 == 0 && Bs->stride[1] % 16 == 0 && ((uintptr_t)Bs->ptr) % 16 == 0 &&
              N * b_ld < ((int64_t)1 << 31) && As->stride[0] % 16 == 0 && ((uintptr_t)As->ptr) % 16 == 0)
       kernel = MX_KERNEL_DECODE;
-    else if (M > 128 && N > 128 && (int64_t)M * N >= (int64_t)1024 * 1024) kernel = MX_KERNEL_MFMA_256x256;
+    else if (M > 128 && N > 128 && (int64_t)M * N >= (int64_t)1024 * 1024) kernel = big_tile_kernel();
     else kernel = MX_KERNEL_MFMA_128x128;
   } else if (kernel != MX_KERNEL_GENERIC && why) {
     return set_error(MX_ERR_LAYOUT, "requested kernel %d cannot run this problem: %s", kernel, why);
@@ -367,7 +375,7 @@ int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W,
   int kernel = o.kernel;
   if (kernel == MX_KERNEL_AUTO) {
     if (why) kernel = MX_KERNEL_GENERIC;
-    else kernel = (tile_m % 256 == 0 && N > 128) ? MX_KERNEL_MFMA_256x256 : MX_KERNEL_MFMA_128x128;
+    else kernel = (tile_m % 256 == 0 && N > 128) ? big_tile_kernel() : MX_KERNEL_MFMA_128x128;
   } else if (kernel != MX_KERNEL_GENERIC) {
     if (why) return set_error(MX_ERR_LAYOUT, "requested kernel %d cannot run this problem: %s", kernel, why);
     const int bm = kernel == MX_KERNEL_MFMA_128x128 ? 128 : 256;

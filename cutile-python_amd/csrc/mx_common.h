@@ -98,6 +98,7 @@ struct GemmArgs {
 };
 
 int launch_gemm_mfma(const GemmArgs& g, int kernel_id, hipStream_t stream);
+int launch_gemm_pingpong(const GemmArgs& g, hipStream_t stream);
 
 struct GenericArgs {
   const uint8_t* A; const uint8_t* As; const uint8_t* B; const uint8_t* Bs; void* C;

@@ -91,7 +91,8 @@ enum {
   MX_KERNEL_MFMA_128x128 = 2, /* v_mfma_scale tiles, 128x128 macro tile, 4 waves                */
   MX_KERNEL_MFMA_256x256 = 3, /* 256x256 macro tile, 8 waves                                    */
   MX_KERNEL_MFMA_256x256_W4 = 4, /* 256x256 macro tile, 4 waves                                 */
-  MX_KERNEL_DECODE = 5        /* skinny-M (M <= 32) weight-streaming kernel                     */
+  MX_KERNEL_DECODE = 5,       /* skinny-M (M <= 32) weight-streaming kernel                     */
+  MX_KERNEL_MFMA_PINGPONG = 6 /* 256x256 macro tile, two 4-wave teams alternating LDS/MFMA phases */
 };
 
 typedef struct mx_gemm_opts {

@@ -70,7 +70,7 @@ def _moe_case(T, K, N, E, topk, seed, dev, w_std=0.1):
 
 
 @pytest.mark.parametrize("kernel,tile", [("generic", 16), ("generic", 128), ("mfma128", 128), ("mfma128", 256),
-                                         ("mfma256", 256), ("mfma256w4", 256), ("auto", 128), ("auto", 256)])
+                                         ("mfma256", 256), ("mfma256w4", 256), ("pingpong", 256), ("auto", 128), ("auto", 256)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=str)
 def test_grouped_gemm_sample_shape(ct, dev, kernel, tile, out_dtype):
     """samples/MoE.py:420-462 shape: 48 tokens, hidden 512, 64 experts, top-8; N = 1024."""

@@ -9,7 +9,7 @@ from oracle import mx_oracle as O
 
 pytestmark = pytest.mark.gpu
 TOL = {torch.float32: 1e-3, torch.bfloat16: 8e-3}
-MFMA = ["mfma128", "mfma256", "mfma256w4"]
+MFMA = ["mfma128", "mfma256", "mfma256w4", "pingpong"]
 
 
 def _run(ct, a: Operand, b: Operand, **kw):
