@@ -1,4 +1,4 @@
-// Ping-pong block-scaled GEMM for large problems (gfx950): 256 x 256 tile, 8 waves.
+// Persistent ping-pong block-scaled GEMM for large problems (gfx950): 256 x 256 tile, 8 waves.
 //
 // Same math, operand layouts and LDS swizzle as the kernel in mx_gemm_mfma.hip; what differs is the
 // schedule.  The 8 waves form two teams of four (one wave of each team per SIMD): team 0 owns rows
@@ -20,6 +20,13 @@
 //           read) for stage s + 2 into the buffer of stage s, right after its own reads of stage s;
 //           wave (0, wn) read them one phase earlier and will read the new contents three phases
 //           later, behind the barrier at which team 1 waits for the loads (vmcnt).
+//
+// Persistence: a workgroup walks a list of tiles.  The stage pipeline runs straight across tile
+// boundaries (the last two stages of a tile prefetch the first two of the next one), and the output
+// of a finished tile is converted and stored inside the first memory phase of the next tile, i.e.
+// while the other team is in an MFMA phase, so neither the pipeline fill nor the epilogue idles the
+// matrix pipe.  A workgroup is given more than one tile only when a tile has at least two stages and
+// a whole number of K-quads (K a multiple of 512).
 #include <stdlib.h>
 
 #include <type_traits>
@@ -43,9 +50,49 @@ struct PP {
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
-template <class C, typename OutT, bool GROUPED, int TEAM>
+// Output of a tile that touches the matrix edge, accumulates into C or has an unaligned C: every
+// element checked.  Deliberately not inlined (the accumulators are passed by value) so that its address
+// arithmetic and branches stay out of the register allocation of the main loop.
+struct AccTile {
+  v4f v[8][4];
+};
+
+template <typename OutT>
+__device__ __attribute__((noinline)) void write_tile_checked(AccTile t, OutT* Cp, int64_t ldc, int M, int N,
+                                                             int mw, int nw, bool accumulate,
+                                                             bool vec_ok) {
+  // mw / nw: row of the lane in tile (0, j) / first column of the lane in tile (i, 0)
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m = mw + 16 * i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = nw + 16 * j;
+      if (n >= N) continue;
+      store4<OutT>(Cp + (int64_t)m * ldc + n, t.v[i][j], accumulate, N - n, vec_ok);
+    }
+  }
+}
+
+// Tiles a workgroup walks: linear tile ids first, first + step, ... below end.  Linear ids map to
+// (tile row, tile column) in groups of 8 tile rows walked column by column (L2 reuse of the B columns).
+struct TileWalk {
+  int first, step, end, tiles_m, tiles_n;
+  __device__ void origin(int lid, int& m0, int& n0) const {
+    constexpr int GM = 8;
+    const int in_group = GM * tiles_n;
+    const int gid = lid / in_group, first_m = gid * GM;
+    const int gsz = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
+    const int in = lid % in_group;
+    m0 = (first_m + in % gsz) * 256;
+    n0 = (in / gsz) * 256;
+  }
+};
+
+template <class C, typename OutT, bool GROUPED, int TEAM, int VAR>
 __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, const int wn,
-                                        const int lane, const int m0, const int n0) {
+                                        const int lane, const TileWalk& walk) {
   using P = PP<C>;
   constexpr int AL = P::AL, BL = P::BL;
   const int r = lane & 15, gq = lane >> 4;
@@ -56,14 +103,16 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   const int ksteps = (g.K + 127) / 128;
   const int nstages = (ksteps + C::KSUB - 1) / C::KSUB;
   const int KQ = (ksteps + 3) / 4;
-
-  int expert = 0;
-  if constexpr (GROUPED) expert = g.sorted_expert_ids[m0 / g.tile_m];
-  const uint8_t* Bbase = g.B + (GROUPED ? (int64_t)expert * g.b_expert_stride : 0);
+  const int a_groups = (g.M + 63) / 64, b_groups = (g.N + 63) / 64;
+  // K rotation: this workgroup walks the K-quads of every tile starting at quad rotQ (whole quads only)
+  int rotQ = 0;
+  if (g.stagger && ksteps % 4 == 0)
+    rotQ = (int)(((blockIdx.x & 7) * (g.stagger & 0xFF) +
+                  ((blockIdx.x >> 3) % (((g.stagger >> 16) & 0xFF) + 1)) * ((g.stagger >> 8) & 0xFF)) % KQ);
+  const int rotS = rotQ * (4 / C::KSUB);
   const __amdgpu_buffer_rsrc_t rsA = make_rsrc(g.A, (uint32_t)(g.a_rows * g.lda));
-  const __amdgpu_buffer_rsrc_t rsB = make_rsrc(Bbase, (uint32_t)((int64_t)g.N * g.ldb));
 
-  // ---- DMA work of this lane -----------------------------------------------------------------------
+  // ---- load context: where the DMA and scale loads of the tile being FETCHED point --------------------
   // A: instruction q of the wave covers tile rows wm0 + (4 q + wn) * A_RPI ...; B (team 1 only):
   // rows wn0 + q * B_RPI ....  The swizzled byte column of instruction q is col0 ^ (4 q % CPR) * 16.
   uint32_t a_voff[AL], b_voff[TEAM ? BL : 1];
@@ -71,70 +120,86 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   const int a_col0 = ((lane % C::A_CPR) ^ swz<C::A_CPR>(a_row0)) * 16;
   const int b_row0 = wn0 + lane / C::B_CPR;
   const int b_col0 = ((lane % C::B_CPR) ^ swz<C::B_CPR>(b_row0)) * 16;
-#pragma unroll
-  for (int q = 0; q < AL; ++q) {
-    const int col = a_col0 ^ (((4 * q * 4) % C::A_CPR) << 4);
-    int64_t grow = m0 + a_row0 + q * 4 * P::A_RPI;
-    bool ok = grow < g.M;
-    if constexpr (GROUPED) {
-      const int id = ok ? g.sorted_token_ids[grow] : 0x7FFFFFFF;
-      ok = ok && id >= 0 && id < g.num_valid_ids;
-      grow = id / g.replicas;
-    }
-    a_voff[q] = ok ? (uint32_t)(grow * g.lda + col) : kOobOffset;
-  }
-  if constexpr (TEAM == 1) {
-#pragma unroll
-    for (int q = 0; q < BL; ++q) {
-      const int col = b_col0 ^ (((4 * q) % C::B_CPR) << 4);
-      const int64_t grow = n0 + b_row0 + q * P::B_RPI;
-      b_voff[q] = grow < g.N ? (uint32_t)(grow * g.ldb + col) : kOobOffset;
-    }
-  }
-  // stage s of A into buffer abuf; a stage at or beyond nstages, and the 16-byte chunks beyond the end
-  // of K, read nothing and zero-fill their LDS bytes (out-of-range buffer offset)
-  auto issue_a = [&](int s, int abuf) {
-    lds_u8* const base = smem + abuf * C::A_STAGE + wm0 * C::A_RB + wn * 1024;
-    const int ka = s * C::A_RB;
-    const int klim = s < nstages ? Kb_a - ka : 0;   // bytes of this stage's rows that exist
+  __amdgpu_buffer_rsrc_t rsB;
+  // scale groups (16-byte index of K-quad 0, lane 0) of this wave's rows / columns: for the tile being
+  // computed and for the tile being fetched
+  int as_cur[2], bs_cur, as_nxt[2], bs_nxt;
+  const v4i* const As4 = (const v4i*)g.As + lane;
+  const v4i* const Bs4 = (const v4i*)g.Bs + lane;
+  bool fetch_valid = true;   // false once the walk has no further tile: loads become zero-fill no-ops
+  auto set_fetch_tile = [&](int lid) {
+    fetch_valid = lid < walk.end;
+    int m0 = 0, n0 = 0;
+    if (fetch_valid) walk.origin(lid, m0, n0);
+    int expert = 0;
+    if constexpr (GROUPED) expert = g.sorted_expert_ids[m0 / g.tile_m];
+    const uint8_t* Bbase = g.B + (GROUPED ? (int64_t)expert * g.b_expert_stride : 0);
+    rsB = make_rsrc(Bbase, (uint32_t)((int64_t)g.N * g.ldb));
 #pragma unroll
     for (int q = 0; q < AL; ++q) {
-      const int col = a_col0 ^ (((4 * q * 4) % C::A_CPR) << 4);
-      const uint32_t v = col >= klim ? kOobOffset : a_voff[q];
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_void*)(base + q * 4096), 16, v, ka, 0, 0);
+      int64_t grow = m0 + a_row0 + q * 4 * P::A_RPI;
+      bool ok = fetch_valid && grow < g.M;
+      if constexpr (GROUPED) {
+        const int id = ok ? g.sorted_token_ids[grow] : 0x7FFFFFFF;
+        ok = ok && id >= 0 && id < g.num_valid_ids;
+        grow = id / g.replicas;
+      }
+      a_voff[q] = ok ? (uint32_t)(grow * g.lda + a_col0) : kOobOffset;
+    }
+    if constexpr (TEAM == 1) {
+#pragma unroll
+      for (int q = 0; q < BL; ++q) {
+        const int col = b_col0 ^ (((4 * q) % C::B_CPR) << 4);
+        const int64_t grow = n0 + b_row0 + q * P::B_RPI;
+        b_voff[q] = (fetch_valid && grow < g.N) ? (uint32_t)(grow * g.ldb + col) : kOobOffset;
+      }
+    }
+    // a tile that overhangs the matrix reuses the last scale group (its rows are discarded anyway)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int grp = (m0 + wm0) / 64 + u;
+      as_nxt[u] = (grp < a_groups ? grp : a_groups - 1) * KQ * 64;
+    }
+    const int grp = (n0 + wn0) / 64;
+    bs_nxt = (GROUPED ? (int)(expert * (g.bs_expert_stride / 4)) : 0) +
+             (grp < b_groups ? grp : b_groups - 1) * KQ * 64;
+  };
+  // local stage sl of the fetch tile into A buffer abuf / B buffer bbuf; a stage at or beyond nstages
+  // and the 16-byte chunks beyond the end of K read nothing and zero-fill their LDS bytes
+  // (out-of-range buffer offset)
+  auto issue_a = [&](int sl, int abuf) {
+    if constexpr (VAR & 1) return;
+    lds_u8* const base = smem + abuf * C::A_STAGE + wm0 * C::A_RB + wn * 1024;
+    int sk = sl + rotS;
+    if (sk >= nstages && sl < nstages) sk -= nstages;
+    if constexpr (VAR & 8) sk &= 3;   // timing aid: every stage re-reads the first four (cache-resident)
+    const int ka = sk * C::A_RB;
+    const int klim = sl < nstages ? Kb_a - ka : 0;   // bytes of this stage's rows that exist
+#pragma unroll
+    for (int q = 0; q < AL; ++q) {
+      const uint32_t v = a_col0 >= klim ? kOobOffset : a_voff[q];
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_void*)(base + q * 4096), 16, v, ka, 0, (VAR >> 8));
     }
   };
-  auto issue_b = [&](int s, int bbuf) {
+  auto issue_b = [&](int sl, int bbuf) {
+    if constexpr (VAR & 1) return;
     if constexpr (TEAM == 1) {
       lds_u8* const base = smem + P::B_BASE + bbuf * C::B_STAGE + wn0 * C::B_RB;
-      const int kb = s * C::B_RB;
-      const int klim = s < nstages ? Kb_b - kb : 0;
+      int sk = sl + rotS;
+      if (sk >= nstages && sl < nstages) sk -= nstages;
+      if constexpr (VAR & 8) sk &= 3;
+      const int kb = sk * C::B_RB;
+      const int klim = sl < nstages ? Kb_b - kb : 0;
 #pragma unroll
       for (int q = 0; q < BL; ++q) {
         const int col = b_col0 ^ (((4 * q) % C::B_CPR) << 4);
         const uint32_t v = col >= klim ? kOobOffset : b_voff[q];
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(base + q * 1024), 16, v, kb, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(base + q * 1024), 16, v, kb, 0, (VAR >> 8));
       }
     }
   };
 
-  // ---- scales (native layout): one 16-byte load per 64-row group and K-quad ---------------------------
-  const v4i* const as_ptr = (const v4i*)g.As + lane;
-  const v4i* const bs_ptr =
-      (const v4i*)(g.Bs + (GROUPED ? (int64_t)expert * g.bs_expert_stride : 0)) + lane;
-  const int a_groups = (g.M + 63) / 64, b_groups = (g.N + 63) / 64;
-  int64_t a_sidx[2], b_sidx;   // a tile that overhangs the matrix reuses the last group (rows discarded)
-#pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const int grp = (m0 + wm0) / 64 + u;
-    a_sidx[u] = (int64_t)(grp < a_groups ? grp : a_groups - 1) * KQ * 64;
-  }
-  {
-    const int grp = (n0 + wn0) / 64;
-    b_sidx = (int64_t)(grp < b_groups ? grp : b_groups - 1) * KQ * 64;
-  }
   v4i sa[2], sb;
-
   v4f acc[8][4];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
@@ -143,14 +208,74 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   const int swa = swz<C::A_CPR>(r), swb = swz<C::B_CPR>(r);
   constexpr int SPQ = 4 / C::KSUB;   // stages per K-quad
 
-  // ---- prologue: stages 0 and 1, scales of quad 0 -----------------------------------------------------
+  // ---- output of a finished tile: lane (c, g) of tile (i, j) holds rows 16 i + c, columns
+  // 16 j + 4 g .. + 3; the accumulators are cleared for the next tile ------------------------------------
+  OutT* const Cp = (OutT*)g.C;
+  const bool vec_ok = (g.ldc % 4 == 0) && (((uintptr_t)g.C) % 16 == 0);
+  const bool accumulate = g.accumulate != 0;
+  auto write_tile = [&](int m0, int n0) {
+    if constexpr (!GROUPED) {
+      // interior tile, plain store: one address per lane, everything else immediate offsets
+      if (m0 + 256 <= g.M && n0 + 256 <= g.N && vec_ok && !accumulate) {
+        OutT* p = Cp + (int64_t)(m0 + wm0 + r) * g.ldc + (n0 + wn0 + 4 * gq);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (!(VAR & 2) || g.ldc == -12345) store4_full<OutT>(p + 16 * j, acc[i][j]);
+            acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+          }
+          p += 16 * g.ldc;
+        }
+        return;
+      }
+      AccTile t;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          t.v[i][j] = acc[i][j];
+          acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+        }
+      if (!(VAR & 2) || g.ldc == -12345)
+        write_tile_checked<OutT>(t, Cp, g.ldc, g.M, g.N, m0 + wm0 + r, n0 + wn0 + 4 * gq, accumulate, vec_ok);
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int m = m0 + wm0 + 16 * i + r;
+      int64_t orow = m;
+      bool ok = m < g.M;
+      float w = 1.f;
+      if constexpr (GROUPED) {
+        const int id = ok ? g.sorted_token_ids[m] : 0x7FFFFFFF;
+        ok = ok && id >= 0 && id < g.num_valid_ids;
+        orow = id;
+        if (ok && g.topk_weights) w = g.topk_weights[id];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + wn0 + 16 * j + 4 * gq;
+        if ((!(VAR & 2) || g.ldc == -12345) && ok && n < g.N) {
+          v4f v = acc[i][j];
+          if constexpr (GROUPED) v *= w;
+          store4<OutT>(Cp + orow * g.ldc + n, v, accumulate, g.N - n, vec_ok);
+        }
+        acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+      }
+    }
+  };
+
+  // ---- prologue: stages 0 and 1 of the first tile, scales of its K-quad 0 ---------------------------------
+  int lid = walk.first;          // tile being computed
+  set_fetch_tile(lid);
   issue_a(0, 0);
   issue_b(0, 0);
   issue_a(1, 1);
   issue_b(1, 1);
 #pragma unroll
-  for (int u = 0; u < 2; ++u) sa[u] = as_ptr[a_sidx[u]];
-  sb = bs_ptr[b_sidx];
+  for (int u = 0; u < 2; ++u) sa[u] = As4[as_nxt[u] + rotQ * 64];
+  sb = Bs4[bs_nxt + rotQ * 64];
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_barrier" ::: "memory");
@@ -164,9 +289,22 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     const int s = Q * SPQ + t0 / C::KSUB;
     if (s >= nstages) return;
     // =============================== memory phase ==================================================
+    if constexpr (t0 == 0) {
+      if (s == 0 && lid != walk.first) {
+        // the previous tile's output leaves while the other team is in its MFMA phase
+        int pm0, pn0;
+        walk.origin(lid - walk.step, pm0, pn0);
+        write_tile(pm0, pn0);
+      }
+    }
+    // from stage nstages - 2 on, the loads run ahead into the next tile of the walk
+    if (s + 2 == nstages) set_fetch_tile(lid + walk.step);
+    const bool wrapped = s + 2 >= nstages;
+    const int sl = wrapped ? s + 2 - nstages : s + 2;   // local stage the loads fetch
+    const int sl_eff = (wrapped && (!fetch_valid || nstages < 2)) ? nstages : sl;
     lds_u8* const atile = smem + abuf * C::A_STAGE + (wm0 + r) * C::A_RB;
     lds_u8* const btile = smem + P::B_BASE + bbuf * C::B_STAGE + (wn0 + r) * C::B_RB;
-    issue_a(s + 2, abuf2);
+    issue_a(sl_eff, abuf2);
     v8i bf[C::KSUB][4], af[C::KSUB][8];
 #pragma unroll
     for (int kk = 0; kk < C::KSUB; ++kk) {
@@ -179,9 +317,9 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       // the B buffer of this stage is free once this wave's own reads have returned
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
-      issue_b(s + 2, bbuf);
+      issue_b(sl_eff, bbuf);
       // everything older than this phase's loads has landed: A and B of stage s + 1
-      __builtin_amdgcn_s_waitcnt(0x0F70 | (AL + BL));
+      if constexpr (!(VAR & 1)) __builtin_amdgcn_s_waitcnt(0x0F70 | (AL + BL));
     }
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // fragments are in registers
@@ -194,8 +332,10 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
 #pragma unroll
         for (int kk = 0; kk < C::KSUB; ++kk)
 #pragma unroll
-          for (int i = 2 * ip + 2; i < 2 * ip + 4; ++i)
-            af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
+          for (int i = 2 * ip + 2; i < 2 * ip + 4; ++i) {
+            if constexpr (VAR & 4) af[kk][i] = af[kk][i & 1];
+            else af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
+          }
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -219,15 +359,18 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     }
     constexpr bool last_of_quad = (t0 + C::KSUB == 4);
     if constexpr (last_of_quad) {
-      // scales of the next quad; they travel during the barrier and the next memory phase
-      const int Qn = Q + 1 < KQ ? Q + 1 : Q;
+      // scales of the next K-quad (quad 0 of the tile being fetched after the last quad); they travel
+      // during the barrier and the next memory phase
+      const bool more = Q + 1 < KQ;
+      int Qk = (more ? Q + 1 : 0) + rotQ;
+      if (Qk >= KQ) Qk -= KQ;
 #pragma unroll
-      for (int u = 0; u < 2; ++u) sa[u] = as_ptr[a_sidx[u] + (int64_t)Qn * 64];
-      sb = bs_ptr[b_sidx + (int64_t)Qn * 64];
+      for (int u = 0; u < 2; ++u) sa[u] = As4[(more ? as_cur[u] : as_nxt[u]) + Qk * 64];
+      sb = Bs4[(more ? bs_cur : bs_nxt) + Qk * 64];
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (TEAM == 0) {
+    if constexpr (TEAM == 0 && !(VAR & 1)) {
       // A of stage s + 1 (issued one stage ago) must have landed; A of stage s + 2 and the scale
       // loads just issued may stay in flight
       __builtin_amdgcn_s_waitcnt(0x0F70 | (AL + (last_of_quad ? P::SCALE_LOADS : 0)));
@@ -238,77 +381,69 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     abuf2 = abuf2 == 2 ? 0 : abuf2 + 1;
     bbuf ^= 1;
   };
-  for (Q = 0; Q < KQ; ++Q) {
-    stage(std::integral_constant<int, 0>{});
-    if constexpr (C::KSUB == 1) stage(std::integral_constant<int, 1>{});
-    stage(std::integral_constant<int, 2>{});
-    if constexpr (C::KSUB == 1) stage(std::integral_constant<int, 3>{});
+  for (; lid < walk.end; lid += walk.step) {
+    as_cur[0] = as_nxt[0];
+    as_cur[1] = as_nxt[1];
+    bs_cur = bs_nxt;
+    for (Q = 0; Q < KQ; ++Q) {
+      stage(std::integral_constant<int, 0>{});
+      if constexpr (C::KSUB == 1) stage(std::integral_constant<int, 1>{});
+      stage(std::integral_constant<int, 2>{});
+      if constexpr (C::KSUB == 1) stage(std::integral_constant<int, 3>{});
+    }
   }
-  if constexpr (TEAM == 0) asm volatile("s_barrier" ::: "memory");   // pairs with team 1's extra barrier
   __builtin_amdgcn_s_waitcnt(0x0F70);   // trailing zero-fill DMA has left the queue
   __builtin_amdgcn_sched_barrier(0);
-
-  // ---- epilogue: lane (c, g) of tile (i, j) holds rows 16 i + c, columns 16 j + 4 g .. + 3 -------------
-  OutT* const Cp = (OutT*)g.C;
-  const bool vec_ok = (g.ldc % 4 == 0) && (((uintptr_t)g.C) % 16 == 0);
-  const bool accumulate = g.accumulate != 0;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int m = m0 + wm0 + 16 * i + r;
-    int64_t orow = m;
-    bool ok = m < g.M;
-    float w = 1.f;
-    if constexpr (GROUPED) {
-      const int id = ok ? g.sorted_token_ids[m] : 0x7FFFFFFF;
-      ok = ok && id >= 0 && id < g.num_valid_ids;
-      orow = id;
-      if (ok && g.topk_weights) w = g.topk_weights[id];
-    }
-    if (!ok) continue;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int n = n0 + wn0 + 16 * j + 4 * gq;
-      if (n >= g.N) continue;
-      v4f v = acc[i][j];
-      if constexpr (GROUPED) v *= w;
-      store4<OutT>(Cp + orow * g.ldc + n, v, accumulate, g.N - n, vec_ok);
-    }
+  {
+    int pm0, pn0;
+    walk.origin(lid - walk.step, pm0, pn0);
+    write_tile(pm0, pn0);
   }
+  if constexpr (TEAM == 0) asm volatile("s_barrier" ::: "memory");   // pairs with team 1's extra barrier
 }
 
-template <class C, typename OutT, bool GROUPED>
+template <class C, typename OutT, bool GROUPED, int VAR>
 __global__ __launch_bounds__(512) void gemm_pp_kernel(const GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
   lds_u8* const smem = (lds_u8*)smem_generic;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
-  // XCD-aware tile order (workgroup ids are dealt round-robin to the 8 XCDs: give each XCD a
-  // contiguous range of tiles), then groups of 8 tile rows walked column by column for L2 reuse
-  const int tiles_m = (g.M + 255) / 256, tiles_n = (g.N + 255) / 256;
-  int tile_m, tile_n;
+  // Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2): XCD x owns a contiguous
+  // range of linear tile ids, and its workgroups walk that range with a stride of their count.
+  TileWalk walk;
+  walk.tiles_m = (g.M + 255) / 256;
+  walk.tiles_n = (g.N + 255) / 256;
   {
-    const int total = tiles_m * tiles_n;
-    const int pid = blockIdx.x;
+    const int total = walk.tiles_m * walk.tiles_n;
+    const int pid = blockIdx.x, grid = gridDim.x;
     const int xcd = pid & 7, loc = pid >> 3, per = total >> 3, rem = total & 7;
-    const int lid = xcd * per + (xcd < rem ? xcd : rem) + loc;
-    constexpr int GM = 8;
-    const int in_group = GM * tiles_n;
-    const int gid = lid / in_group, first_m = gid * GM;
-    const int gsz = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
-    const int in = lid % in_group;
-    tile_m = first_m + in % gsz;
-    tile_n = in / gsz;
+    const int start = xcd * per + (xcd < rem ? xcd : rem);
+    const int count = per + (xcd < rem ? 1 : 0);
+    walk.step = (grid - xcd + 7) >> 3;   // workgroups of this XCD
+    walk.first = start + loc;
+    walk.end = start + count;
   }
+  if (walk.first >= walk.end) return;   // cannot happen with the grids the launcher picks
   if (wave < 4)
-    pp_body<C, OutT, GROUPED, 0>(g, smem, wave, lane, tile_m * 256, tile_n * 256);
+    pp_body<C, OutT, GROUPED, 0, VAR>(g, smem, wave, lane, walk);
   else
-    pp_body<C, OutT, GROUPED, 1>(g, smem, wave - 4, lane, tile_m * 256, tile_n * 256);
+    pp_body<C, OutT, GROUPED, 1, VAR>(g, smem, wave - 4, lane, walk);
 }
 
-template <class C, typename OutT, bool GROUPED>
+int num_cus() {
+  static int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+    return n;
+  }();
+  return cus;
+}
+
+template <class C, typename OutT, bool GROUPED, int VAR = 0>
 int launch_pp(const GemmArgs& g, hipStream_t stream) {
-  auto kern = gemm_pp_kernel<C, OutT, GROUPED>;
+  auto kern = gemm_pp_kernel<C, OutT, GROUPED, VAR>;
   static int attr_done = 0;   // benign race: the attribute call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -320,7 +455,15 @@ int launch_pp(const GemmArgs& g, hipStream_t stream) {
   }
   const int64_t tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
   if (tiles <= 0) return MX_OK;
-  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(512), PP<C>::LDS_BYTES, stream, g);
+  // one workgroup per CU walking several tiles when the stage pipeline can run across tile boundaries
+  // (at least two stages per tile, whole K-quads); otherwise one workgroup per tile
+  const int ksteps = (g.K + 127) / 128;
+  const int nstages = (ksteps + C::KSUB - 1) / C::KSUB;
+  const bool can_walk = nstages >= 2 && ksteps % 4 == 0;
+  static const int walk_env = [] { const char* e = getenv("MXGEMM_PP_WALK"); return e ? atoi(e) : 1; }();
+  int64_t grid = tiles;
+  if (can_walk && walk_env && tiles > num_cus()) grid = num_cus();
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), PP<C>::LDS_BYTES, stream, g);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "gemm_pp_kernel launch: %s", hipGetErrorString(e));
   return MX_OK;
@@ -328,10 +471,35 @@ int launch_pp(const GemmArgs& g, hipStream_t stream) {
 
 }  // namespace
 
-int launch_gemm_pingpong(const GemmArgs& g, hipStream_t stream) {
-  if (g.c_dtype != MX_F32 && g.c_dtype != MX_BF16)
-    return set_error(MX_ERR_DTYPE, "MFMA kernel: output dtype %d not supported", g.c_dtype);
-  const bool grouped = g.sorted_token_ids != nullptr;
+int launch_gemm_pingpong(const GemmArgs& g0, hipStream_t stream) {
+  if (g0.c_dtype != MX_F32 && g0.c_dtype != MX_BF16)
+    return set_error(MX_ERR_DTYPE, "MFMA kernel: output dtype %d not supported", g0.c_dtype);
+  const bool grouped = g0.sorted_token_ids != nullptr;
+  static const int rot_env = [] { const char* e = getenv("MXGEMM_PP_ROT"); return e ? (int)strtol(e, nullptr, 0) : 0; }();
+  GemmArgs gr = g0;
+  gr.stagger = rot_env;
+  const GemmArgs& g = gr;
+  // timing aids (MXGEMM_PP_VAR, read once): 1 no DMA in the loop, 2 no output stores, 4 no late LDS reads
+  static const int var_env = [] { const char* e = getenv("MXGEMM_PP_VAR"); return e ? (int)strtol(e, nullptr, 0) : 0; }();
+  if (var_env && g.a_fmt == MX_E4M3 && g.b_fmt == MX_E4M3 && g.c_dtype == MX_BF16 && !grouped) {
+    using C = Cfg<MX_E4M3, MX_E4M3, 256, 256, 2, 4>;
+    switch (var_env) {
+      case 1: return launch_pp<C, uint16_t, false, 1>(g, stream);
+      case 2: return launch_pp<C, uint16_t, false, 2>(g, stream);
+      case 3: return launch_pp<C, uint16_t, false, 3>(g, stream);
+      case 4: return launch_pp<C, uint16_t, false, 4>(g, stream);
+      case 5: return launch_pp<C, uint16_t, false, 5>(g, stream);
+      case 7: return launch_pp<C, uint16_t, false, 7>(g, stream);
+      case 8: return launch_pp<C, uint16_t, false, 8>(g, stream);
+      case 10: return launch_pp<C, uint16_t, false, 10>(g, stream);
+      case 0x100: return launch_pp<C, uint16_t, false, 0x100>(g, stream);
+      case 0x200: return launch_pp<C, uint16_t, false, 0x200>(g, stream);
+      case 0x300: return launch_pp<C, uint16_t, false, 0x300>(g, stream);
+      case 0x1000: return launch_pp<C, uint16_t, false, 0x1000>(g, stream);
+      case 0x1100: return launch_pp<C, uint16_t, false, 0x1100>(g, stream);
+      case 0x1200: return launch_pp<C, uint16_t, false, 0x1200>(g, stream);
+    }
+  }
 #define MX_CASE(AFMT, BFMT)                                                                        \
   if (g.a_fmt == AFMT && g.b_fmt == BFMT) {                                                        \
     using C = Cfg<AFMT, BFMT, 256, 256, 2, 4>;                                                     \

@@ -103,4 +103,24 @@ __device__ inline void store4<uint16_t>(uint16_t* p, const v4f& v, bool accumula
   }
 }
 
+// four consecutive outputs, no bounds, alignment or accumulate handling (interior tiles)
+template <typename OutT>
+__device__ inline void store4_full(OutT* p, const v4f& v);
+
+template <>
+__device__ inline void store4_full<float>(float* p, const v4f& v) {
+  *(v4f*)p = v;
+}
+
+template <>
+__device__ inline void store4_full<uint16_t>(uint16_t* p, const v4f& v) {
+  // v_cvt_pk_bf16_f32: round to nearest even, the same result as f32_to_bf16 for every non-NaN input
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  uint2 w;
+  w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v.x, v.y}, b2));
+  w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v.z, v.w}, b2));
+  *(uint2*)p = w;
+}
+
 }  // namespace mx
