@@ -4,10 +4,10 @@
 // schedule.  The 8 waves form two teams of four (one wave of each team per SIMD): team 0 owns rows
 // 0-127 of the tile, team 1 rows 128-255; wave (team, wn) computes the 128 x 64 block at columns
 // 64 wn.  Every K stage of a wave is split into
-//   a MEMORY phase: LDS-DMA issue for stage s + 2, LDS reads of the B fragments and the first two A
+//   a MEMORY phase: LDS-DMA issue for stage s + 2, LDS reads of the B fragments and the first A
 //                   tiles of stage s;
 //   an MFMA phase:  32 (64 for FP4) back-to-back MFMAs from registers, with the reads of the other
-//                   six A tiles slotted in two tiles ahead of their use.
+//                   remaining A tiles slotted in 8 or 16 MFMAs ahead of their use.
 // One s_barrier ends every phase.  Team 1 runs exactly one phase behind team 0 (it executes one extra
 // barrier before its first stage, team 0 one extra after its last), so the two waves of a SIMD are
 // never in the same phase: while one waits on LDS, issues DMA or sits in a barrier, the other feeds
@@ -35,6 +35,9 @@
 
 namespace mx {
 namespace {
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
+constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 
 template <class C>
 struct PP {
@@ -95,6 +98,9 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
                                         const int lane, const TileWalk& walk) {
   using P = PP<C>;
   constexpr int AL = P::AL, BL = P::BL;
+  // A tiles (of 8) whose fragments are read in the memory phase; the gather / scatter bookkeeping of the
+  // grouped variant leaves registers for two only
+  constexpr int EARLY = GROUPED ? 2 : 4;
   const int r = lane & 15, gq = lane >> 4;
   constexpr int wm0 = TEAM * 128;
   const int wn0 = wn * 64;
@@ -104,12 +110,6 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   const int nstages = (ksteps + C::KSUB - 1) / C::KSUB;
   const int KQ = (ksteps + 3) / 4;
   const int a_groups = (g.M + 63) / 64, b_groups = (g.N + 63) / 64;
-  // K rotation: this workgroup walks the K-quads of every tile starting at quad rotQ (whole quads only)
-  int rotQ = 0;
-  if (g.stagger && ksteps % 4 == 0)
-    rotQ = (int)(((blockIdx.x & 7) * (g.stagger & 0xFF) +
-                  ((blockIdx.x >> 3) % (((g.stagger >> 16) & 0xFF) + 1)) * ((g.stagger >> 8) & 0xFF)) % KQ);
-  const int rotS = rotQ * (4 / C::KSUB);
   const __amdgpu_buffer_rsrc_t rsA = make_rsrc(g.A, (uint32_t)(g.a_rows * g.lda));
 
   // ---- load context: where the DMA and scale loads of the tile being FETCHED point --------------------
@@ -170,23 +170,21 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   auto issue_a = [&](int sl, int abuf) {
     if constexpr (VAR & 1) return;
     lds_u8* const base = smem + abuf * C::A_STAGE + wm0 * C::A_RB + wn * 1024;
-    int sk = sl + rotS;
-    if (sk >= nstages && sl < nstages) sk -= nstages;
+    int sk = sl;
     if constexpr (VAR & 8) sk &= 3;   // timing aid: every stage re-reads the first four (cache-resident)
     const int ka = sk * C::A_RB;
     const int klim = sl < nstages ? Kb_a - ka : 0;   // bytes of this stage's rows that exist
 #pragma unroll
     for (int q = 0; q < AL; ++q) {
       const uint32_t v = a_col0 >= klim ? kOobOffset : a_voff[q];
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_void*)(base + q * 4096), 16, v, ka, 0, (VAR >> 8));
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_void*)(base + q * 4096), 16, v, ka, 0, 0);
     }
   };
   auto issue_b = [&](int sl, int bbuf) {
     if constexpr (VAR & 1) return;
     if constexpr (TEAM == 1) {
       lds_u8* const base = smem + P::B_BASE + bbuf * C::B_STAGE + wn0 * C::B_RB;
-      int sk = sl + rotS;
-      if (sk >= nstages && sl < nstages) sk -= nstages;
+      int sk = sl;
       if constexpr (VAR & 8) sk &= 3;
       const int kb = sk * C::B_RB;
       const int klim = sl < nstages ? Kb_b - kb : 0;
@@ -194,7 +192,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       for (int q = 0; q < BL; ++q) {
         const int col = b_col0 ^ (((4 * q) % C::B_CPR) << 4);
         const uint32_t v = col >= klim ? kOobOffset : b_voff[q];
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(base + q * 1024), 16, v, kb, 0, (VAR >> 8));
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(base + q * 1024), 16, v, kb, 0, 0);
       }
     }
   };
@@ -274,8 +272,8 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   issue_a(1, 1);
   issue_b(1, 1);
 #pragma unroll
-  for (int u = 0; u < 2; ++u) sa[u] = As4[as_nxt[u] + rotQ * 64];
-  sb = Bs4[bs_nxt + rotQ * 64];
+  for (int u = 0; u < 2; ++u) sa[u] = As4[as_nxt[u]];
+  sb = Bs4[bs_nxt];
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_barrier" ::: "memory");
@@ -311,7 +309,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
 #pragma unroll
       for (int j = 0; j < 4; ++j) bf[kk][j] = load_frag<C::B_RB, C::B_EB>(btile, 16 * j, kk, gq, swb);
 #pragma unroll
-      for (int i = 0; i < 2; ++i) af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
+      for (int i = 0; i < EARLY; ++i) af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
     }
     if constexpr (TEAM == 1) {
       // the B buffer of this stage is free once this wave's own reads have returned
@@ -319,29 +317,31 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       __builtin_amdgcn_sched_barrier(0);
       issue_b(sl_eff, bbuf);
       // everything older than this phase's loads has landed: A and B of stage s + 1
-      if constexpr (!(VAR & 1)) __builtin_amdgcn_s_waitcnt(0x0F70 | (AL + BL));
+      // (the scale loads issued at the end of the previous quad are younger than those and may stay in
+      // flight; the MFMA phase waits for them)
+      constexpr int younger = (t0 == 0) ? P::SCALE_LOADS : 0;
+      if constexpr (!(VAR & 1)) __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL + BL + younger));
     }
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // fragments are in registers
     __builtin_amdgcn_sched_barrier(0);
     // =============================== MFMA phase ====================================================
     __builtin_amdgcn_s_setprio(1);
+    auto read_pair = [&](int i0) {
 #pragma unroll
-    for (int ip = 0; ip < 4; ++ip) {   // pairs of A tiles
-      if (ip < 3) {
+      for (int kk = 0; kk < C::KSUB; ++kk)
 #pragma unroll
-        for (int kk = 0; kk < C::KSUB; ++kk)
-#pragma unroll
-          for (int i = 2 * ip + 2; i < 2 * ip + 4; ++i) {
-            if constexpr (VAR & 4) af[kk][i] = af[kk][i & 1];
-            else af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
-          }
-      }
+        for (int i = i0; i < i0 + 2; ++i) {
+          if constexpr (VAR & 4) af[kk][i] = af[kk][i & 1];
+          else af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
+        }
       __builtin_amdgcn_sched_barrier(0);
+    };
+    auto mfma_pair = [&](int i0) {
 #pragma unroll
       for (int kk = 0; kk < C::KSUB; ++kk) {
 #pragma unroll
-        for (int i = 2 * ip; i < 2 * ip + 2; ++i) {
+        for (int i = i0; i < i0 + 2; ++i) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             if (t0 + kk == 0)
@@ -356,14 +356,19 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+    };
+    // A tiles below EARLY were read in the memory phase; the rest is read EARLY * 4 MFMAs ahead of use
+#pragma unroll
+    for (int ip = 0; ip < 8; ip += 2) {
+      if (ip + EARLY < 8) read_pair(ip + EARLY);
+      mfma_pair(ip);
     }
     constexpr bool last_of_quad = (t0 + C::KSUB == 4);
     if constexpr (last_of_quad) {
       // scales of the next K-quad (quad 0 of the tile being fetched after the last quad); they travel
       // during the barrier and the next memory phase
       const bool more = Q + 1 < KQ;
-      int Qk = (more ? Q + 1 : 0) + rotQ;
-      if (Qk >= KQ) Qk -= KQ;
+      const int Qk = more ? Q + 1 : 0;
 #pragma unroll
       for (int u = 0; u < 2; ++u) sa[u] = As4[(more ? as_cur[u] : as_nxt[u]) + Qk * 64];
       sb = Bs4[(more ? bs_cur : bs_nxt) + Qk * 64];
@@ -373,7 +378,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     if constexpr (TEAM == 0 && !(VAR & 1)) {
       // A of stage s + 1 (issued one stage ago) must have landed; A of stage s + 2 and the scale
       // loads just issued may stay in flight
-      __builtin_amdgcn_s_waitcnt(0x0F70 | (AL + (last_of_quad ? P::SCALE_LOADS : 0)));
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL + (last_of_quad ? P::SCALE_LOADS : 0)));
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
@@ -471,14 +476,10 @@ int launch_pp(const GemmArgs& g, hipStream_t stream) {
 
 }  // namespace
 
-int launch_gemm_pingpong(const GemmArgs& g0, hipStream_t stream) {
-  if (g0.c_dtype != MX_F32 && g0.c_dtype != MX_BF16)
-    return set_error(MX_ERR_DTYPE, "MFMA kernel: output dtype %d not supported", g0.c_dtype);
-  const bool grouped = g0.sorted_token_ids != nullptr;
-  static const int rot_env = [] { const char* e = getenv("MXGEMM_PP_ROT"); return e ? (int)strtol(e, nullptr, 0) : 0; }();
-  GemmArgs gr = g0;
-  gr.stagger = rot_env;
-  const GemmArgs& g = gr;
+int launch_gemm_pingpong(const GemmArgs& g, hipStream_t stream) {
+  if (g.c_dtype != MX_F32 && g.c_dtype != MX_BF16)
+    return set_error(MX_ERR_DTYPE, "MFMA kernel: output dtype %d not supported", g.c_dtype);
+  const bool grouped = g.sorted_token_ids != nullptr;
   // timing aids (MXGEMM_PP_VAR, read once): 1 no DMA in the loop, 2 no output stores, 4 no late LDS reads
   static const int var_env = [] { const char* e = getenv("MXGEMM_PP_VAR"); return e ? (int)strtol(e, nullptr, 0) : 0; }();
   if (var_env && g.a_fmt == MX_E4M3 && g.b_fmt == MX_E4M3 && g.c_dtype == MX_BF16 && !grouped) {
@@ -492,12 +493,6 @@ int launch_gemm_pingpong(const GemmArgs& g0, hipStream_t stream) {
       case 7: return launch_pp<C, uint16_t, false, 7>(g, stream);
       case 8: return launch_pp<C, uint16_t, false, 8>(g, stream);
       case 10: return launch_pp<C, uint16_t, false, 10>(g, stream);
-      case 0x100: return launch_pp<C, uint16_t, false, 0x100>(g, stream);
-      case 0x200: return launch_pp<C, uint16_t, false, 0x200>(g, stream);
-      case 0x300: return launch_pp<C, uint16_t, false, 0x300>(g, stream);
-      case 0x1000: return launch_pp<C, uint16_t, false, 0x1000>(g, stream);
-      case 0x1100: return launch_pp<C, uint16_t, false, 0x1100>(g, stream);
-      case 0x1200: return launch_pp<C, uint16_t, false, 0x1200>(g, stream);
     }
   }
 #define MX_CASE(AFMT, BFMT)                                                                        \
