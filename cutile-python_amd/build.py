@@ -28,7 +28,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hi
 def _newer(src: pathlib.Path, obj: pathlib.Path) -> bool:
     if not obj.exists():
         return True
-    deps = [src, CSRC / "mx_common.h", INCLUDE / "mxgemm.h"]
+    deps = [src, CSRC / "mx_common.h", CSRC / "mx_gemm_tile.h", INCLUDE / "mxgemm.h"]
     return any(d.stat().st_mtime > obj.stat().st_mtime for d in deps)
 
 

@@ -108,13 +108,14 @@ int64_t mx_gemm_grouped_workspace_bytes(int64_t num_slots, int64_t N, int64_t K,
   return b;
 }
 
-int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, void* packed,
-                   void* stream) {
+namespace {
+// validates a scale tensor against (rows, K) and describes its re-layout into `packed`
+int make_pack_args(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, void* packed, PackArgs& p) {
   if (int rc = check_tensor(scale, "scale", 2, 4)) return rc;
   if (!packed) return set_error(MX_ERR_INVALID, "packed: null pointer");
   if (K % 32 != 0) return set_error(MX_ERR_SHAPE, "K (%lld) must be a multiple of 32", (long long)K);
   if (((uintptr_t)packed) % 16 != 0) return set_error(MX_ERR_LAYOUT, "packed buffer must be 16-byte aligned");
-  PackArgs p = {};
+  p = PackArgs{};
   p.src = (const uint8_t*)scale->ptr;
   p.dst = (uint32_t*)packed;
   p.rows = rows;
@@ -148,6 +149,14 @@ int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t
   } else {
     return set_error(MX_ERR_INVALID, "mx_pack_scales: unknown source layout %d", layout);
   }
+  return MX_OK;
+}
+}  // namespace
+
+int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, void* packed,
+                   void* stream) {
+  PackArgs p;
+  if (int rc = make_pack_args(scale, layout, rows, K, packed, p)) return rc;
   return launch_pack_scales(p, (hipStream_t)stream);
 }
 
@@ -300,20 +309,24 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
     return set_error(MX_ERR_WORKSPACE, "workspace must be 256-byte aligned");
   const uint32_t* as_native = (const uint32_t*)As->ptr;
   const uint32_t* bs_native = (const uint32_t*)Bs->ptr;
-  if (o.a_scale_layout != MX_SCALE_NATIVE) {
-    if (int rc = mx_pack_scales(As, o.a_scale_layout, M, K, ws, stream)) return rc;
+  PackArgs pa, pb;
+  const bool pack_a = o.a_scale_layout != MX_SCALE_NATIVE, pack_b = o.b_scale_layout != MX_SCALE_NATIVE;
+  if (pack_a) {
+    if (int rc = make_pack_args(As, o.a_scale_layout, M, K, ws, pa)) return rc;
     as_native = (const uint32_t*)ws;
     ws += mx_packed_scale_bytes(M, K);
   }
-  if (o.b_scale_layout != MX_SCALE_NATIVE) {
+  if (pack_b) {
     mx_tensor t = *Bs;
     if (o.b_scale_layout == MX_SCALE_2D) {  // [K/32, N] -> view as [N, K/32]
       t.shape[0] = Bs->shape[1]; t.shape[1] = Bs->shape[0];
       t.stride[0] = Bs->stride[1]; t.stride[1] = Bs->stride[0];
     }
-    if (int rc = mx_pack_scales(&t, o.b_scale_layout, N, K, ws, stream)) return rc;
+    if (int rc = make_pack_args(&t, o.b_scale_layout, N, K, ws, pb)) return rc;
     bs_native = (const uint32_t*)ws;
   }
+  if (pack_a || pack_b)   // one launch for both operands
+    if (int rc = launch_pack_scales_pair(pack_a ? &pa : nullptr, pack_b ? &pb : nullptr, (hipStream_t)stream)) return rc;
   if (((uintptr_t)as_native) % 16 != 0 || ((uintptr_t)bs_native) % 16 != 0)
     return set_error(MX_ERR_LAYOUT, "native scale buffers must be 16-byte aligned");
 
@@ -408,23 +421,22 @@ int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W,
     return set_error(MX_ERR_WORKSPACE, "workspace of %lld bytes required, %lld given", (long long)need,
                      (long long)workspace_bytes);
   if (((uintptr_t)ws) % 256 != 0) return set_error(MX_ERR_WORKSPACE, "workspace must be 256-byte aligned");
-  // A scales: gathered into slot order while re-laying
-  {
-    PackArgs p = {};
-    p.src = (const uint8_t*)As->ptr; p.dst = (uint32_t*)ws;
-    p.rows = num_slots; p.K = K; p.s_row = As->stride[0]; p.s_kb = As->stride[1];
-    p.layout = MX_SCALE_2D; p.batch = 1;
-    p.gather_ids = sorted_token_ids; p.replicas = num_token_replicas; p.num_valid_ids = num_valid_ids;
-    if (int rc = launch_pack_scales(p, (hipStream_t)stream)) return rc;
-  }
+  // A scales: gathered into slot order while re-laying; W scales of all experts ride in the same launch
+  PackArgs pa = {}, pw;
+  pa.src = (const uint8_t*)As->ptr; pa.dst = (uint32_t*)ws;
+  pa.rows = num_slots; pa.K = K; pa.s_row = As->stride[0]; pa.s_kb = As->stride[1];
+  pa.layout = MX_SCALE_2D; pa.batch = 1;
+  pa.gather_ids = sorted_token_ids; pa.replicas = num_token_replicas; pa.num_valid_ids = num_valid_ids;
   const uint32_t* as_native = (const uint32_t*)ws;
   ws += mx_packed_scale_bytes(num_slots, K);
   const uint32_t* bs_native = (const uint32_t*)Ws->ptr;
-  if (o.b_scale_layout != MX_SCALE_NATIVE) {
+  const bool pack_w = o.b_scale_layout != MX_SCALE_NATIVE;
+  if (pack_w) {
     if (o.b_scale_layout != MX_SCALE_2D) return set_error(MX_ERR_LAYOUT, "W_scale must be [E, N, K/32] or native");
-    if (int rc = mx_pack_scales(Ws, MX_SCALE_2D, N, K, ws, stream)) return rc;
+    if (int rc = make_pack_args(Ws, MX_SCALE_2D, N, K, ws, pw)) return rc;
     bs_native = (const uint32_t*)ws;
   }
+  if (int rc = launch_pack_scales_pair(&pa, pack_w ? &pw : nullptr, (hipStream_t)stream)) return rc;
   GemmArgs g = {};
   g.A = (const uint8_t*)A->ptr; g.B = (const uint8_t*)W->ptr; g.As = as_native; g.Bs = bs_native; g.C = C->ptr;
   g.lda = A->stride[0]; g.ldb = W->stride[1]; g.ldc = C->stride[0];

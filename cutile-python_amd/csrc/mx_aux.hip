@@ -173,42 +173,86 @@ __global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
 // ================================================================================================
 // Native scale re-layout (see mx_common.h for the layout)
 // ================================================================================================
-__global__ __launch_bounds__(256) void pack_scales_kernel(const PackArgs p) {
+// One workgroup re-lays out 64 rows x 4 K-quads (64 scale bytes per row) of one operand: the bytes are
+// staged in LDS with whichever axis is contiguous in the source mapped to consecutive lanes (16-byte
+// loads when alignment allows), then every thread assembles the four dwords of one (quad, lane) and
+// writes them with one 16-byte store.  Up to two operands (A and B scales of one GEMM) share a launch.
+struct PackPair {
+  PackArgs p[2];
+  int32_t blocks0;   // workgroups that belong to p[0]
+};
+
+__device__ inline int64_t scale_src_offset(const PackArgs& p, int64_t srow, int64_t kb, int64_t KB) {
+  if (p.layout == MX_SCALE_SWIZZLE_32_4_4) {
+    const int64_t m0 = srow >> 7, m2 = (srow & 127) >> 5, m1 = srow & 31, k0 = kb >> 2, k1 = kb & 3;
+    return ((m0 * (KB >> 2) + k0) * 32 + m1) * 16 + m2 * 4 + k1;
+  }
+  return srow * p.s_row + kb * p.s_kb;
+}
+
+__global__ __launch_bounds__(256) void pack_scales_kernel(const PackPair pp) {
+  constexpr int LD = 68;   // LDS row pitch (bytes): 64 scale bytes + 4 so that rows start on distinct banks
+  __shared__ __attribute__((aligned(16))) uint8_t tile[64 * LD];
+  const bool second = (int)blockIdx.x >= pp.blocks0;
+  const PackArgs& p = second ? pp.p[1] : pp.p[0];
+  const int64_t blk = second ? blockIdx.x - pp.blocks0 : blockIdx.x;
   const int64_t KB = p.K / 32;
   const int64_t KQ = packed_scale_quads(p.K);
-  const int64_t per_batch = packed_scale_dwords(p.rows, p.K);
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= per_batch) return;
-  const int64_t b = blockIdx.y;
-  const int i4 = (int)(idx & 3), lane = (int)((idx >> 2) & 63);
-  const int64_t Q = (idx >> 8) % KQ, t64 = (idx >> 8) / KQ;
-  const int64_t row = t64 * 64 + i4 * 16 + (lane & 15);
-  const int g = lane >> 4;
+  const int64_t qgroups = (KQ + 3) / 4, rgroups = (p.rows + 63) / 64;
+  const int64_t b = blk / (qgroups * rgroups);
+  const int64_t t64 = (blk / qgroups) % rgroups;
+  const int64_t Q0 = (blk % qgroups) * 4;
+  const int tid = threadIdx.x;
+  const uint8_t* src = p.src + b * p.s_batch;
+  const int64_t row0 = t64 * 64, kb0 = Q0 * 16;
 
-  int64_t srow = row;
-  bool ok = row < p.rows;
-  if (p.gather_ids) {
-    const int id = ok ? p.gather_ids[row] : -1;
-    ok = ok && id >= 0 && id < p.num_valid_ids;
-    srow = id / p.replicas;
-  }
-  uint32_t out = 0;
-  for (int t = 0; t < 4; ++t) {
-    const int64_t kb = (Q * 4 + t) * 4 + g;
-    uint32_t byte = 127;  // 1.0 for padding: multiplies zero-filled operand data
-    if (ok && kb < KB) {
-      int64_t off;
-      if (p.layout == MX_SCALE_SWIZZLE_32_4_4) {
-        const int64_t m0 = srow >> 7, m2 = (srow & 127) >> 5, m1 = srow & 31, k0 = kb >> 2, k1 = kb & 3;
-        off = ((m0 * (KB >> 2) + k0) * 32 + m1) * 16 + m2 * 4 + k1;
-      } else {
-        off = srow * p.s_row + kb * p.s_kb;
-      }
-      byte = p.src[b * p.s_batch + off];
+  // ---- stage 64 rows x 64 scale bytes; 127 (1.0) wherever the source has nothing -------------------------
+  const bool plain = p.layout == MX_SCALE_2D && !p.gather_ids;
+  if (plain && p.s_row == 1 && p.s_kb != 1) {
+    // rows contiguous in the source: thread = (kb, 16 consecutive rows)
+    const int kbi = tid >> 2, c = tid & 3;
+    const int64_t kb = kb0 + kbi, r0 = row0 + c * 16;
+    alignas(16) uint8_t v[16];
+    const uint8_t* s = src + kb * p.s_kb + r0;
+    if (kb < KB && r0 + 16 <= p.rows && (((uintptr_t)s) & 15) == 0) {
+      *(uint4*)v = *(const uint4*)s;
+    } else {
+      for (int e = 0; e < 16; ++e) v[e] = (kb < KB && r0 + e < p.rows) ? s[e] : 127;
     }
-    out |= byte << (8 * t);
+    for (int e = 0; e < 16; ++e) tile[(c * 16 + e) * LD + kbi] = v[e];
+  } else {
+    // thread = (row, 16 consecutive K blocks)
+    const int rowi = tid >> 2, c = tid & 3;
+    const int64_t row = row0 + rowi, kb = kb0 + c * 16;
+    int64_t srow = row;
+    bool ok = row < p.rows;
+    if (p.gather_ids) {
+      const int id = ok ? p.gather_ids[row] : -1;
+      ok = ok && id >= 0 && id < p.num_valid_ids;
+      srow = id / p.replicas;
+    }
+    alignas(16) uint8_t v[16];
+    const uint8_t* s = src + srow * p.s_row + kb;
+    if (ok && p.layout == MX_SCALE_2D && p.s_kb == 1 && kb + 16 <= KB && (((uintptr_t)s) & 15) == 0) {
+      *(uint4*)v = *(const uint4*)s;
+    } else {
+      for (int e = 0; e < 16; ++e) v[e] = (ok && kb + e < KB) ? src[scale_src_offset(p, srow, kb + e, KB)] : 127;
+    }
+    *(uint4*)(tile + rowi * LD + c * 16) = *(const uint4*)v;
   }
-  p.dst[b * per_batch + idx] = out;
+  __syncthreads();
+
+  // ---- assemble: thread = (quad q of the group, lane); dword i4 = row 16 i4 + lane % 16, byte t =
+  // K block (4 (Q0 + q) + t) * 4 + lane / 16 -----------------------------------------------------------------
+  const int q = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+  if (Q0 + q >= KQ) return;
+  uint32_t out[4];
+  for (int i4 = 0; i4 < 4; ++i4) {
+    const uint8_t* t = tile + (i4 * 16 + r) * LD + q * 16 + g;
+    out[i4] = (uint32_t)t[0] | ((uint32_t)t[4] << 8) | ((uint32_t)t[8] << 16) | ((uint32_t)t[12] << 24);
+  }
+  uint32_t* dst = p.dst + b * packed_scale_dwords(p.rows, p.K) + ((t64 * KQ + Q0 + q) * 64 + lane) * 4;
+  *(uint4*)dst = make_uint4(out[0], out[1], out[2], out[3]);
 }
 
 // ================================================================================================
@@ -279,6 +323,74 @@ __global__ __launch_bounds__(256) void moe_align_kernel(const int32_t* __restric
   }
 }
 
+// Parallel variant for E <= 256 experts: every thread owns a contiguous segment of the ids.
+//   1. per-thread, per-expert counts (LDS, u16, one column per thread: no atomics);
+//   2. thread e turns row e into exclusive prefixes over the threads (earlier segments come first, which is
+//      what makes the sort stable) and keeps the expert's total;
+//   3. exclusive scan of the tile-padded totals over the experts;
+//   4. every thread places its segment in order at start[e] + prefix[e][thread]++;
+//   5. padding slots get the sentinel n, blocks get their expert.  No slot is written twice.
+__global__ __launch_bounds__(256) void moe_align_seg_kernel(const int32_t* __restrict__ topk_ids, int64_t n,
+                                                            int32_t E, int32_t tile_m,
+                                                            int32_t* __restrict__ sorted_ids,
+                                                            int32_t* __restrict__ expert_ids,
+                                                            int32_t* __restrict__ num_slots_out,
+                                                            int64_t max_slots) {
+  constexpr int T = 256, LD = T + 2;   // row pitch 129 dwords: rows start on consecutive LDS banks
+  extern __shared__ int32_t sh[];
+  int32_t* total = sh;                  // [E] ids per expert
+  int32_t* start = sh + E;              // [E + 1] first slot of each expert
+  uint16_t* cnt = (uint16_t*)(sh + 2 * E + 2);   // [E][LD]
+  const int tid = threadIdx.x;
+  const int64_t seg = (n + T - 1) / T;
+  const int64_t lo = tid * seg < n ? tid * seg : n, hi = lo + seg < n ? lo + seg : n;
+  for (int i = tid; i < E * LD / 2; i += T) ((uint32_t*)cnt)[i] = 0;
+  __syncthreads();
+  for (int64_t i = lo; i < hi; ++i) {
+    const int e = topk_ids[i];
+    if (e >= 0 && e < E) cnt[e * LD + tid] += 1;
+  }
+  __syncthreads();
+  if (tid < E) {
+    uint16_t* row = cnt + tid * LD;
+    int32_t run = 0;
+    for (int t = 0; t < T; ++t) {
+      const int32_t c = row[t];
+      row[t] = (uint16_t)run;
+      run += c;
+    }
+    total[tid] = run;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int32_t s = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = s;
+      s += (total[e] + tile_m - 1) / tile_m * tile_m;
+    }
+    start[E] = s;
+    if (num_slots_out) *num_slots_out = s;
+  }
+  __syncthreads();
+  for (int64_t i = lo; i < hi; ++i) {
+    const int e = topk_ids[i];
+    if (e >= 0 && e < E) {
+      const int32_t pos = start[e] + cnt[e * LD + tid];
+      cnt[e * LD + tid] += 1;
+      sorted_ids[pos] = (int32_t)i;
+    }
+  }
+  // padding behind every expert's ids, the unused tail, and the block -> expert map (trailing unused
+  // blocks name expert 0; their slots hold the sentinel)
+  for (int e = tid; e < E; e += T) {
+    for (int32_t s2 = start[e] + total[e]; s2 < start[e + 1]; ++s2) sorted_ids[s2] = (int32_t)n;
+    for (int32_t s2 = start[e]; s2 < start[e + 1]; s2 += tile_m) expert_ids[s2 / tile_m] = e;
+  }
+  const int32_t used = start[E];
+  for (int64_t i = used + tid; i < max_slots; i += T) sorted_ids[i] = (int32_t)n;
+  for (int64_t blk = used / tile_m + tid; blk < max_slots / tile_m; blk += T) expert_ids[blk] = 0;
+}
+
 }  // namespace
 
 int launch_quantize(const QuantArgs& q, hipStream_t stream) {
@@ -292,23 +404,52 @@ int launch_quantize(const QuantArgs& q, hipStream_t stream) {
   return MX_OK;
 }
 
-int launch_pack_scales(const PackArgs& p, hipStream_t stream) {
-  const int64_t per_batch = packed_scale_dwords(p.rows, p.K);
-  if (per_batch <= 0 || p.batch <= 0) return MX_OK;
-  dim3 grid((unsigned)((per_batch + 255) / 256), (unsigned)p.batch);
-  hipLaunchKernelGGL(pack_scales_kernel, grid, dim3(256), 0, stream, p);
+int launch_pack_scales_pair(const PackArgs* a, const PackArgs* b, hipStream_t stream) {
+  PackPair pp = {};
+  int64_t blocks[2] = {0, 0};
+  const PackArgs* ops[2] = {a, b};
+  int n = 0;
+  for (int i = 0; i < 2; ++i) {
+    const PackArgs* p = ops[i];
+    if (!p || p->rows <= 0 || p->K <= 0 || p->batch <= 0) continue;
+    pp.p[n] = *p;
+    blocks[n] = ((p->rows + 63) / 64) * ((packed_scale_quads(p->K) + 3) / 4) * p->batch;
+    ++n;
+  }
+  if (n == 0) return MX_OK;
+  const int64_t total = blocks[0] + blocks[1];
+  if (total > 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "pack_scales: tensor too large");
+  pp.blocks0 = (int32_t)blocks[0];
+  hipLaunchKernelGGL(pack_scales_kernel, dim3((unsigned)total), dim3(256), 0, stream, pp);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "pack_scales_kernel launch: %s", hipGetErrorString(e));
   return MX_OK;
 }
 
+int launch_pack_scales(const PackArgs& p, hipStream_t stream) {
+  return launch_pack_scales_pair(&p, nullptr, stream);
+}
+
 int launch_moe_align(const int32_t* topk_ids, int64_t num_ids, int32_t num_experts, int32_t tile_m,
                      int32_t* sorted_token_ids, int32_t* sorted_expert_ids, int32_t* num_slots_out,
                      int64_t max_slots, hipStream_t stream) {
-  const size_t lds = (size_t)(2 * num_experts + 1) * sizeof(int32_t);
-  if (lds > 60000) return set_error(MX_ERR_SHAPE, "moe_align: too many experts (%d)", num_experts);
-  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(256), lds, stream, topk_ids, num_ids, num_experts,
-                     tile_m, sorted_token_ids, sorted_expert_ids, num_slots_out, max_slots);
+  if (num_experts <= 256 && num_ids <= (int64_t)256 * 65535) {
+    const size_t lds = (size_t)(2 * num_experts + 2) * sizeof(int32_t) + (size_t)num_experts * 258 * sizeof(uint16_t);
+    static int attr_done = 0;   // benign race: the attribute call is idempotent
+    if (!attr_done) {
+      hipError_t e = hipFuncSetAttribute((const void*)moe_align_seg_kernel,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "hipFuncSetAttribute(moe_align): %s", hipGetErrorString(e));
+      attr_done = 1;
+    }
+    hipLaunchKernelGGL(moe_align_seg_kernel, dim3(1), dim3(256), lds, stream, topk_ids, num_ids, num_experts,
+                       tile_m, sorted_token_ids, sorted_expert_ids, num_slots_out, max_slots);
+  } else {
+    const size_t lds = (size_t)(2 * num_experts + 1) * sizeof(int32_t);
+    if (lds > 60000) return set_error(MX_ERR_SHAPE, "moe_align: too many experts (%d)", num_experts);
+    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(256), lds, stream, topk_ids, num_ids, num_experts,
+                       tile_m, sorted_token_ids, sorted_expert_ids, num_slots_out, max_slots);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "moe_align_kernel launch: %s", hipGetErrorString(e));
   return MX_OK;

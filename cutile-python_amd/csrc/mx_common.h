@@ -128,6 +128,8 @@ struct PackArgs {
   const int32_t* gather_ids; int32_t replicas; int64_t num_valid_ids;
 };
 int launch_pack_scales(const PackArgs& p, hipStream_t stream);
+// both operands of one GEMM in a single launch; either pointer may be null
+int launch_pack_scales_pair(const PackArgs* a, const PackArgs* b, hipStream_t stream);
 
 struct QuantArgs {
   const void* x; uint8_t* xq; uint8_t* scale;

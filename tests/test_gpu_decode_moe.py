@@ -41,7 +41,8 @@ def test_decode_accumulate(ct, dev):
 
 
 @pytest.mark.parametrize("T,topk,E,tile", [(7, 2, 4, 4), (48, 8, 64, 16), (5, 1, 8, 128), (4096, 2, 8, 256),
-                                           (110, 4, 16, 128), (256, 6, 1408, 128)])
+                                           (110, 4, 16, 128), (256, 6, 1408, 128), (1024, 8, 128, 256), (333, 3, 256, 64),
+                                           (3, 1, 200, 32)])
 def test_moe_align_matches_oracle(ct, dev, T, topk, E, tile):
     """test/kernels/fused_moe.py:113-173; shapes from samples/MoE.py:420-462 and test/bench_moe.py:16-24."""
     g = torch.Generator().manual_seed(T + E)

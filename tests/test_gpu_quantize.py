@@ -119,3 +119,46 @@ def test_swizzle_roundtrip_device(ct, dev):
     sw = ct.swizzle_32_4_4(s)
     assert np.array_equal(sw.cpu().numpy(), O.swizzle_32_4_4(s.cpu().numpy()))
     assert torch.equal(ct.unswizzle_32_4_4(sw), s)
+
+
+def _native_layout(sc: np.ndarray) -> np.ndarray:
+    """The packed layout, restated: dword [I / 4][Q][lane][I % 4] holds, in byte t, the scale of row
+    16 I + lane % 16 for K block (4 Q + t) * 4 + lane / 16; rows padded to 64 and blocks to 16 with 127."""
+    rows, KB = sc.shape
+    R, KQ = -(-rows // 64) * 64, -(-KB // 16)
+    full = np.full((R, KQ * 16), 127, dtype=np.uint8)
+    full[:rows, :KB] = sc
+    out = np.zeros((R // 64, KQ, 64, 4, 4), dtype=np.uint8)   # [I/4][Q][lane][I%4][t]
+    for lane in range(64):
+        r, g = lane % 16, lane // 16
+        for i4 in range(4):
+            for t in range(4):
+                out[:, :, lane, i4, t] = full[i4 * 16 + r::64, :].reshape(R // 64, KQ, 16)[:, :, 4 * t + g]
+    return out.reshape(-1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,KB", [(64, 16), (100, 37), (256, 256), (1, 1), (130, 5)])
+@pytest.mark.parametrize("form", ["row_major", "transposed", "sliced", "batched"])
+def test_pack_scales_layout(ct, dev, rows, KB, form):
+    """mx_pack_scales against a restatement of the layout, for every source form the staging code
+    distinguishes (16-byte loads along K or along rows, misaligned sources, batches)."""
+    rng = np.random.default_rng(rows * 1000 + KB)
+    if form == "batched":
+        sc = rng.integers(0, 255, size=(3, rows, KB), dtype=np.uint8)
+        got = ct.pack_scales(torch.from_numpy(sc).to(dev)).data.cpu().numpy()
+        want = np.concatenate([_native_layout(sc[b]) for b in range(3)])
+    else:
+        sc = rng.integers(0, 255, size=(rows, KB), dtype=np.uint8)
+        if form == "row_major":
+            t = torch.from_numpy(sc).to(dev)
+            got = ct.pack_scales(t).data.cpu().numpy()
+        elif form == "transposed":
+            t = torch.from_numpy(np.ascontiguousarray(sc.T)).to(dev)   # [K/32, rows], as B_scale arrives
+            got = ct.pack_scales(t, transposed=True).data.cpu().numpy()
+        else:
+            big = torch.zeros((rows + 3, KB + 7), dtype=torch.uint8, device=dev)
+            big[1:rows + 1, 3:KB + 3] = torch.from_numpy(sc).to(dev)
+            got = ct.pack_scales(big[1:rows + 1, 3:KB + 3]).data.cpu().numpy()
+        want = _native_layout(sc)
+    assert np.array_equal(got, want)
