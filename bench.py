@@ -34,6 +34,10 @@ import torch  # noqa: E402
 
 PEAK_TFLOPS = {"mxfp8": 5033.0, "mxfp4": 10066.0}   # MI355X dense MFMA peaks (vendor figures)
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the headline GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --only c2 --calib-copy`, each scaled by what the same counter reads for the 256 MiB copy kernel
+# (summary under profiles/): 412266 KiB x 2.0 + 156000 KiB x 1.0
+C2_HBM_TRAFFIC_BYTES = 980532 * 1024
 METRIC = "MX GEMM TFLOP/s (+% MFMA peak) 8192^3 MXFP8/MXFP4; GB/s at M=32 decode"
 
 
@@ -219,34 +223,37 @@ def bench_moe(ct, O, dev, steps, warmup, check):
 
 def cpu_baseline_c2(O, sets, budget_s=12.0):
     """The reference's check (dequantize to fp32, torch matmul; samples/BlockScaledMatMul.py:358-364) timed on
-    the host cores on an N-slice of the headline workload, sized from a probe to about `budget_s`."""
+    the host cores on the leading m x m x K corner of the headline workload, m sized from a probe so that the
+    timed run takes about `budget_s` (the whole workload when the host is fast enough)."""
     a_q, a_s, b_q, b_s, _ = sets[0]
     M, K = a_q.shape
-    a_c, a_sc = a_q.view(torch.uint8).cpu().numpy(), a_s.view(torch.uint8).cpu().numpy()
     cores = os.cpu_count() or 1
     try:
         cores = len(os.sched_getaffinity(0))
     except AttributeError:
         pass
-    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    cores = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
     torch.set_num_threads(cores)
+    a_all, as_all = a_q.view(torch.uint8).cpu().numpy(), a_s.view(torch.uint8).cpu().numpy()
+    b_all, bs_all = b_q.view(torch.uint8).cpu().numpy(), b_s.view(torch.uint8).cpu().numpy()
 
-    def run(n):
-        b_c, b_sc = b_q[:n].view(torch.uint8).cpu().numpy(), b_s[:n].view(torch.uint8).cpu().numpy()
+    def run(m):
         t0 = time.perf_counter()
-        a = O.dequantize(a_c, a_sc, O.E4M3)
-        b = O.dequantize(b_c, b_sc, O.E4M3)
+        a = O.dequantize(a_all[:m], as_all[:m], O.E4M3)
+        b = O.dequantize(b_all[:m], bs_all[:m], O.E4M3)
         c = a @ b.T
         dt = time.perf_counter() - t0
         return dt, float(c[0, 0])
 
-    t_probe, _ = run(64)
-    n = int(min(8192, max(64, 64 * budget_s / max(t_probe, 1e-3) // 64 * 64)))
-    dt, _ = run(n)
-    tflops = 2.0 * M * n * K / dt * 1e-12
+    run(256)                      # first-touch / thread-pool warm-up
+    t_probe, _ = run(1024)
+    m = int(1024 * (budget_s / max(t_probe, 1e-4)) ** 0.5) // 64 * 64
+    m = max(1024, min(M, m))
+    dt, _ = run(m)
+    tflops = 2.0 * m * m * K / dt * 1e-12
     return {"value": tflops, "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"torch dequantize + fp32 matmul of the 8192 x {n} x 8192 column slice of the workload, "
-                      f"{dt:.1f} s wall, one run"}
+            "sample": f"oracle dequantize + fp32 matmul of the leading {m} x {m} x {K} corner of the workload "
+                      f"({2.0 * m * m * K * 1e-12:.2f} TFLOP), {dt:.1f} s wall, one run"}
 
 
 def main():
@@ -262,8 +269,8 @@ def main():
                          "scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        raise SystemExit("bench.py: this build runs on ONE GPU (the path has no cross-GPU exchange: weights "
-                         "would be sharded along N, see DESIGN.md); run with --gpus 1")
+        raise SystemExit("bench.py: this build measures ONE GPU (the path has no cross-GPU exchange; a larger "
+                         "job would shard the weights along N and run this same kernel per GPU); run with --gpus 1")
     if not torch.cuda.is_available():
         raise SystemExit("bench.py: no GPU visible")
     import cutile_amd as ct
@@ -314,8 +321,9 @@ def main():
                        "M": 8192, "N": 8192, "K": 8192, "operand_sets_rotated": 3},
             "rel_fro_vs_oracle": r["rel_fro_vs_oracle"],
             "roofline": {"bound": "mfma", "achieved": r["kernel_tflops"], "peak": PEAK_TFLOPS["mxfp8"],
-                         "unit": "TFLOP/s", "frac": r["kernel_tflops"] / PEAK_TFLOPS["mxfp8"], "traffic": None,
-                         "kernel": "gemm_kernel<Cfg<e4m3,e4m3,256,256,2,4>,bf16>", "kernel_ms": r["kernel_ms"],
+                         "unit": "TFLOP/s", "frac": r["kernel_tflops"] / PEAK_TFLOPS["mxfp8"],
+                         "traffic": C2_HBM_TRAFFIC_BYTES,
+                         "kernel": "gemm_pp_kernel<Cfg<e4m3,e4m3,256,256,2,4>,bf16>", "kernel_ms": r["kernel_ms"],
                          "flops_per_launch": r["flops"]},
         })
         if not a.no_cpu:
