@@ -99,40 +99,50 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
   const int t_end = t_begin + per + (b < rem ? 1 : 0);
   if (t_begin >= t_end) return;                // uniform per workgroup
 
-  // The W stream starts before anything else is requested: the first two tiles of this workgroup.
-  MX_ISSUE_TILE(t_begin, 0);
-  if (t_begin + 1 < t_end) MX_ISSUE_TILE(t_begin + 1, 1);
-
   // ---- resident X fragments and scales ---------------------------------------------------------------
-  // All loads are issued unconditionally from clamped addresses (no branches, so they overlap); rows
-  // beyond M and K-steps beyond K are zeroed afterwards.
+  // All loads are issued unconditionally from clamped addresses (no branches, so they overlap), and
+  // before the W stream; they are put into operand form after the first W tiles have been requested.
   v8i xf[MT][SPW];
   int xs[MT][(SPW + 3) / 4];
+  v4i xlo[MT][SPW], xhi[MT][SPW], xsraw[MT][(SPW + 3) / 4];
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
     const int m = 16 * i + r;
     const bool mok = m < d.M;
     const uint8_t* const xrow = d.X + (int64_t)(mok ? m : 0) * d.ldx + gq * 16;
     const uint8_t* const xsrow = d.Xs + (int64_t)(mok ? m : 0) * d.ldxs;
-    v4i lo[SPW], hi[SPW], sraw[(SPW + 3) / 4];
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
       const int ks = s0 + s < ksteps ? s0 + s : 0;
-      if constexpr ((VAR & 4) != 0) { lo[s] = (v4i){s, 1, 2, 3}; hi[s] = lo[s]; continue; }
-      lo[s] = *(const v4i*)(xrow + (int64_t)ks * 128);
-      hi[s] = *(const v4i*)(xrow + (int64_t)ks * 128 + 64);
+      if constexpr ((VAR & 4) != 0) { xlo[i][s] = (v4i){s, 1, 2, 3}; xhi[i][s] = xlo[i][s]; continue; }
+      xlo[i][s] = *(const v4i*)(xrow + (int64_t)ks * 128);
+      xhi[i][s] = *(const v4i*)(xrow + (int64_t)ks * 128 + 64);
     }
 #pragma unroll
     for (int u = 0; u < (SPW + 3) / 4; ++u) {
       // 16 scale bytes = the 4 blocks of K-steps s0 + 4u .. s0 + 4u + 3 (K is a multiple of 512)
       const int ks = s0 + 4 * u < ksteps ? s0 + 4 * u : 0;
-      sraw[u] = *(const v4i*)(xsrow + ks * 4);
+      xsraw[i][u] = *(const v4i*)(xsrow + ks * 4);
     }
+  }
+
+  // The X loads above are requested first: they are few, and queued behind the first W tiles they would
+  // hold back the first MFMA for as long as that burst takes to drain.  Now the W stream starts: the first
+  // two tiles of this workgroup.
+  __builtin_amdgcn_sched_barrier(0);
+  MX_ISSUE_TILE(t_begin, 0);
+  if (t_begin + 1 < t_end) MX_ISSUE_TILE(t_begin + 1, 1);
+
+  __builtin_amdgcn_sched_barrier(0);
+  // X into the MFMA operand layout; rows beyond M and K-steps beyond K become zeros (scale 1.0)
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const bool mok = 16 * i + r < d.M;
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
       const bool ok = mok && s0 + s < ksteps;
-      xf[i][s] = ok ? (v8i){lo[s].x, lo[s].y, lo[s].z, lo[s].w, hi[s].x, hi[s].y, hi[s].z, hi[s].w}
-                    : (v8i){0, 0, 0, 0, 0, 0, 0, 0};
+      const v4i lo = xlo[i][s], hi = xhi[i][s];
+      xf[i][s] = ok ? (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w} : (v8i){0, 0, 0, 0, 0, 0, 0, 0};
     }
 #pragma unroll
     for (int u = 0; u < (SPW + 3) / 4; ++u) {
@@ -140,7 +150,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const bool ok = mok && s0 + 4 * u + t < ksteps;
-        const uint32_t byte = ok ? (((uint32_t)sraw[u][t] >> (8 * gq)) & 0xFFu) : 127u;
+        const uint32_t byte = ok ? (((uint32_t)xsraw[i][u][t] >> (8 * gq)) & 0xFFu) : 127u;
         pk |= byte << (8 * t);
       }
       xs[i][u] = (int)pk;
@@ -162,9 +172,9 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
 #pragma unroll
     for (int i = 0; i < kBatch; ++i) {
       if (i < nt) {                                     // uniform
-        // wait for tile i of the batch; the SPW + 1 loads of tile i + 1 may stay in flight.  (In the very
-        // first iteration the X loads are younger than both tiles: wait for everything.)
-        if (i + 1 < nt && !(i == 0 && tb == t_begin)) __builtin_amdgcn_s_waitcnt(0x0F70 | (SPW + 1));
+        // wait for tile i of the batch (and, the first time, for the older X loads); the SPW + 1 loads of
+        // tile i + 1 may stay in flight
+        if (i + 1 < nt) __builtin_amdgcn_s_waitcnt(0x0F70 | (SPW + 1));
         else __builtin_amdgcn_s_waitcnt(0x0F70);
         asm volatile("" ::: "memory");
         lds_u8* const wt = my + (i & 1) * Cf::SLOT;
