@@ -469,8 +469,10 @@ int mx_moe_align(const int32_t* topk_ids, int64_t num_ids, int32_t num_experts, 
                           num_slots_out, max_slots, (hipStream_t)stream);
 }
 
-int mx_quantize(const mx_tensor* x, mx_tensor* xq, mx_tensor* scale, int32_t scale_mode, void* stream) {
-  if (int rc = check_tensor(x, "x", 2, 2)) return rc;
+namespace {
+// shared by mx_quantize and mx_silu_mul_quantize; K = quantised row length, `up` null for the plain form
+int quantize_common(const mx_tensor* x, const void* up, int64_t K, mx_tensor* xq, mx_tensor* scale,
+                    int32_t scale_mode, void* stream) {
   if (int rc = check_tensor(xq, "xq", 2, 2)) return rc;
   if (int rc = check_tensor(scale, "scale", 2, 2)) return rc;
   if (x->dtype != MX_F32 && x->dtype != MX_BF16 && x->dtype != MX_F16)
@@ -478,7 +480,7 @@ int mx_quantize(const mx_tensor* x, mx_tensor* xq, mx_tensor* scale, int32_t sca
   if (!is_elem(xq->dtype)) return set_error(MX_ERR_DTYPE, "xq must be an MX element format");
   if (scale->dtype != MX_E8M0) return set_error(MX_ERR_DTYPE, "scale must be MX_E8M0");
   if (scale_mode != 0 && scale_mode != 1) return set_error(MX_ERR_INVALID, "scale_mode must be 0 (ceil) or 1 (floor)");
-  const int64_t rows = x->shape[0], K = x->shape[1];
+  const int64_t rows = x->shape[0];
   if (K < 32)
     return set_error(MX_ERR_SHAPE,
                      "The requested block size 32 is larger than the inner most dimension of the input tensor %lld",
@@ -495,7 +497,26 @@ int mx_quantize(const mx_tensor* x, mx_tensor* xq, mx_tensor* scale, int32_t sca
   q.rows = rows; q.K = K; q.Kpad = Kpad;
   q.x_ld = x->stride[0]; q.xq_ld = xq->stride[0]; q.sc_ld = scale->stride[0];
   q.x_dtype = x->dtype; q.fmt = xq->dtype; q.scale_mode = scale_mode;
+  q.up = up;
   return launch_quantize(q, (hipStream_t)stream);
+}
+}  // namespace
+
+int mx_quantize(const mx_tensor* x, mx_tensor* xq, mx_tensor* scale, int32_t scale_mode, void* stream) {
+  if (int rc = check_tensor(x, "x", 2, 2)) return rc;
+  return quantize_common(x, nullptr, x->shape[1], xq, scale, scale_mode, stream);
+}
+
+int mx_silu_mul_quantize(const mx_tensor* gate_up, mx_tensor* xq, mx_tensor* scale, int32_t scale_mode,
+                         void* stream) {
+  if (int rc = check_tensor(gate_up, "gate_up", 2, 2)) return rc;
+  if (gate_up->shape[1] % 2 != 0)
+    return set_error(MX_ERR_SHAPE, "gate_up must have an even number of columns (gate | up), got %lld",
+                     (long long)gate_up->shape[1]);
+  const int64_t F = gate_up->shape[1] / 2;
+  const int esz = gate_up->dtype == MX_F32 ? 4 : 2;
+  const void* up = (const uint8_t*)gate_up->ptr + F * esz;
+  return quantize_common(gate_up, up, F, xq, scale, scale_mode, stream);
 }
 
 }  // extern "C"

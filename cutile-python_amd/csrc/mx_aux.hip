@@ -91,6 +91,43 @@ __device__ inline float load_as_f32(const void* p, int64_t i, int dtype) {
   return (float)((const _Float16*)p)[i];
 }
 
+// silu(a) * b = a / (1 + exp(-a)) * b as a fixed sequence of correctly rounded fp32 operations (no fused
+// multiply-add, no approximate instruction), so that a host restatement with the same sequence gets the
+// same bits: exp(-a) = 2^z, z = -a * log2(e) clamped to +-125, z = n + f with n = rint(z), 2^f by the
+// degree-7 Taylor polynomial in f * ln 2 (|f| <= 0.5: truncation error below 1e-8), scaled by 2^n exactly.
+__device__ inline float silu_mul_f32(float a, float b) {
+  float z = __fmul_rn(-a, 1.44269504f);
+  z = fminf(fmaxf(z, -125.0f), 125.0f);
+  const float n = __builtin_rintf(z);
+  const float f = __fsub_rn(z, n);
+  float p = 1.52527338e-5f;
+  p = __fadd_rn(__fmul_rn(p, f), 1.54035304e-4f);
+  p = __fadd_rn(__fmul_rn(p, f), 1.33335581e-3f);
+  p = __fadd_rn(__fmul_rn(p, f), 9.61812911e-3f);
+  p = __fadd_rn(__fmul_rn(p, f), 5.55041087e-2f);
+  p = __fadd_rn(__fmul_rn(p, f), 2.40226507e-1f);
+  p = __fadd_rn(__fmul_rn(p, f), 6.93147181e-1f);
+  p = __fadd_rn(__fmul_rn(p, f), 1.0f);
+  const float e = __fmul_rn(p, __builtin_bit_cast(float, (uint32_t)((int)n + 127) << 23));
+  const float s = __fdiv_rn(1.0f, __fadd_rn(1.0f, e));
+  const float t = a < -87.5f ? 0.0f : __fmul_rn(a, s);   // exp(-a) is past the clamp: the true value is below 2^-120
+  return __fmul_rn(t, b);
+}
+
+// four consecutive elements starting at element index i (k0 + 3 < K checked by the caller for `vec`)
+__device__ inline void load4_as_f32(const void* p, int64_t i, int dtype, bool vec, int nvalid, float* v) {
+  if (vec && dtype == MX_F32) {
+    const v4f t = *(const v4f*)((const float*)p + i);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  } else if (vec && dtype == MX_BF16) {
+    const uint2 t = *(const uint2*)((const uint16_t*)p + i);
+    v[0] = bf16_to_f32((uint16_t)t.x); v[1] = bf16_to_f32((uint16_t)(t.x >> 16));
+    v[2] = bf16_to_f32((uint16_t)t.y); v[3] = bf16_to_f32((uint16_t)(t.y >> 16));
+  } else {
+    for (int e = 0; e < 4; ++e) v[e] = e < nvalid ? load_as_f32(p, i + e, dtype) : 0.f;
+  }
+}
+
 // 8 lanes per 32-element block, 4 consecutive elements per lane.
 __global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
   const int64_t KB = q.Kpad / 32;
@@ -104,12 +141,15 @@ __global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
   float v[4] = {0.f, 0.f, 0.f, 0.f};
   if (live) {
     const int64_t base = row * q.x_ld + k0;
-    if (q.x_dtype == MX_F32 && k0 + 3 < q.K && ((((uintptr_t)q.x) | (uintptr_t)(q.x_ld * 4)) & 15) == 0) {
-      const v4f t = *(const v4f*)((const float*)q.x + base);
-      v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-    } else {
-      for (int e = 0; e < 4; ++e)
-        if (k0 + e < q.K) v[e] = load_as_f32(q.x, base + e, q.x_dtype);
+    const int esz = q.x_dtype == MX_F32 ? 4 : 2;
+    const int nvalid = q.K - k0 >= 4 ? 4 : (q.K > k0 ? (int)(q.K - k0) : 0);
+    const bool vec = nvalid == 4 && q.x_dtype != MX_F16 &&
+                     ((((uintptr_t)q.x) | ((uintptr_t)q.up) | (uintptr_t)(q.x_ld * esz)) & (4 * esz - 1)) == 0;
+    load4_as_f32(q.x, base, q.x_dtype, vec, nvalid, v);
+    if (q.up) {
+      float u[4];
+      load4_as_f32(q.up, base, q.x_dtype, vec, nvalid, u);
+      for (int e = 0; e < 4; ++e) v[e] = e < nvalid ? silu_mul_f32(v[e], u[e]) : 0.f;
     }
   }
   // amax over the block on |bits| (monotone in |x| for finite values; NaN patterns compare largest)

@@ -136,6 +136,8 @@ struct QuantArgs {
   int64_t rows, K, Kpad;
   int64_t x_ld, xq_ld, sc_ld;    // elements / bytes / bytes
   int32_t x_dtype, fmt, scale_mode;
+  // fused producer: the value quantised is silu(x[row, k]) * up[row, k] (up has the dtype and pitch of x)
+  const void* up;
 };
 int launch_quantize(const QuantArgs& q, hipStream_t stream);
 

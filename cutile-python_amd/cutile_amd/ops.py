@@ -513,3 +513,85 @@ def invoke_fused_moe_scaled(A: torch.Tensor, A_scale: torch.Tensor, B: torch.Ten
                                  ids.numel(), eids.data_ptr(), tile_m, num_token_replicas, num_valid,
                                  ctypes.byref(o), ws.data_ptr(), need, L.stream_ptr(dev))
     _check(rc)
+
+
+def silu_and_mul_quantize(gate_up: torch.Tensor, dtype=torch.float8_e4m3fn, *, scale_mode: str = "floor"):
+    """``silu(gate_up[..., :F]) * gate_up[..., F:]`` MX-quantised along F in blocks of 32, in one pass
+    (the reference runs silu_and_mul_kernel, test/kernels/fused_moe.py:85-108, into a bf16 buffer; here the
+    product never leaves registers before it is quantised).  Returns ``(x_q, scale)`` like
+    :func:`block_quantize`."""
+    if scale_mode not in ("ceil", "floor"):
+        raise TileValueError(f"scale_mode must be 'ceil' or 'floor', got {scale_mode!r}")
+    fmt = dtype if isinstance(dtype, str) else _DTYPE_FMT.get(dtype)
+    if fmt not in _FMT_CODE:
+        raise TileTypeError(f"Unsupported quantisation dtype {dtype}")
+    if gate_up.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        raise TileTypeError(f"Unsupported input dtype {_dtype_name(gate_up.dtype)} for silu_and_mul_quantize")
+    if not gate_up.is_cuda:
+        raise ValueError("Input tensors must be on a CUDA device.")
+    if gate_up.shape[-1] % 2 != 0:
+        raise ValueError("gate_up must have 2 * intermediate_size columns (gate + up projection)")
+    F = gate_up.shape[-1] // 2
+    if F < 32:
+        raise ValueError(f'The requested block size 32 is larger than the inner most '
+                         f'dimension of the input tensor {F}')
+    lead = tuple(gate_up.shape[:-1])
+    x2 = gate_up.reshape(-1, 2 * F)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    Fpad = (F + 31) // 32 * 32
+    if fmt == "e2m1":
+        xq = torch.empty((rows, Fpad // 2), dtype=torch.uint8, device=x2.device)
+        dq = L.desc(xq, L.MX_E2M1, 1)
+    else:
+        xq = torch.empty((rows, Fpad), dtype=torch.uint8, device=x2.device)
+        dq = L.desc(xq, _FMT_CODE[fmt])
+    sc = torch.empty((rows, Fpad // 32), dtype=torch.uint8, device=x2.device)
+    dx = L.desc(x2, L._TORCH_TO_MX[x2.dtype])
+    ds = L.desc(sc, L.MX_E8M0)
+    with torch.cuda.device(x2.device):
+        rc = L.lib().mx_silu_mul_quantize(ctypes.byref(dx), ctypes.byref(dq), ctypes.byref(ds),
+                                          0 if scale_mode == "ceil" else 1, L.stream_ptr(x2.device))
+    _check(rc)
+    if fmt == "e2m1":
+        out = xq.reshape(*lead, Fpad // 2)
+    else:
+        out = xq.view(torch.float8_e4m3fn if fmt == "e4m3" else torch.float8_e5m2).reshape(*lead, Fpad)
+    return out, sc.view(torch.float8_e8m0fnu).reshape(*lead, Fpad // 32)
+
+
+def cutile_moe_scaled(hidden_states: torch.Tensor, hidden_scale: torch.Tensor,
+                      w1: torch.Tensor, w1_scale, w2: torch.Tensor, w2_scale,
+                      topk_weights: torch.Tensor, topk_ids: torch.Tensor, tile_m: int = 256, *,
+                      out_dtype: torch.dtype = torch.bfloat16, scale_mode: str = "floor",
+                      w_format: Optional[str] = None, kernel: str = "auto") -> torch.Tensor:
+    """Block-scaled Mixture-of-Experts forward with the structure of ``cutile_moe``
+    (samples/MoE.py:197-288): align -> grouped gate+up GEMM -> SiLU(gate) * up -> grouped down GEMM
+    with the routed-weight multiply -> sum over the top-k copies.
+
+    hidden_states (tokens, H) MX elements with hidden_scale (tokens, H/32); w1 (E, 2F, H) and w2 (E, H, F)
+    MX elements (FP4 packed along the last axis, ``w_format="e2m1"``) with scales (E, rows, K/32) or
+    :class:`PackedScales`; topk_weights / topk_ids (tokens, topk).  The intermediate activation is
+    re-quantised to E4M3 on the device (one fused pass) so that both GEMMs run block-scaled.  Nothing in the
+    call synchronises with the host.  Returns (tokens, H) in ``out_dtype``."""
+    if hidden_states.dim() != 2 or w1.dim() != 3 or w2.dim() != 3:
+        raise TileTypeError("hidden_states must be 2D, w1 and w2 3D")
+    T = hidden_states.shape[0]
+    E = w1.shape[0]
+    topk = topk_ids.shape[1]
+    two_f = w1.shape[1]
+    H_out = w2.shape[1]
+    if two_f % 2 != 0:
+        raise ValueError("w1 must have 2 * intermediate_size rows (gate + up projection)")
+    dev = hidden_states.device
+    ids, eids = moe_align_tile_size(topk_ids, tile_m, E, exact=False)
+    cache1 = torch.empty((T * topk, two_f), dtype=torch.bfloat16, device=dev)
+    invoke_fused_moe_scaled(hidden_states, hidden_scale, w1, w1_scale, cache1, None, ids, eids, False, topk,
+                            tile_m, b_format=w_format, kernel=kernel)
+    a2, a2s = silu_and_mul_quantize(cache1, torch.float8_e4m3fn, scale_mode=scale_mode)
+    # rows of ids that no expert claimed (ids outside [0, E)) stay zero, as in the reference's zeros() caches
+    cache3 = torch.zeros((T, topk, H_out), dtype=torch.float32, device=dev)
+    invoke_fused_moe_scaled(a2, a2s, w2, w2_scale, cache3, topk_weights, ids, eids, True, 1, tile_m,
+                            b_format=w_format, kernel=kernel)
+    return cache3.sum(dim=1).to(out_dtype)

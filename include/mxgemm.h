@@ -187,6 +187,19 @@ MX_API int mx_quantize(const mx_tensor* x, mx_tensor* xq, mx_tensor* scale, int3
                 void* stream);
 
 /*
+ * Fused activation producer of the MoE pipeline: silu(gate) * up, MX-quantised in one pass (replaces
+ * silu_and_mul_kernel, test/kernels/fused_moe.py:85-108, followed by block_quantize, so that the
+ * down-projection of cutile_moe, samples/MoE.py:197-288, can also run block-scaled).
+ *   gate_up [rows, 2F] MX_F32 | MX_BF16 | MX_F16, last stride 1: gate = [:, :F], up = [:, F:]
+ *   xq      [rows, Fpad] elements, scale [rows, Fpad/32] MX_E8M0, scale_mode: as mx_quantize
+ * The product is formed in fp32 as a fixed sequence of correctly rounded operations
+ * (a / (1 + 2^(-a log2 e)) * b with a degree-7 polynomial for the fractional power), so a host
+ * restatement reproduces it bit for bit; it is within a few 1e-7 relative of torch's silu(a) * b.
+ */
+MX_API int mx_silu_mul_quantize(const mx_tensor* gate_up, mx_tensor* xq, mx_tensor* scale, int32_t scale_mode,
+                         void* stream);
+
+/*
  * Re-lays a scale tensor into the MFMA-ready native layout consumed by the MFMA kernels
  * (no reference counterpart: the reference's swizzle_32_4_4, test/kernels/kernel_utils.py:83-98,
  * is the Blackwell analogue).  `scale` is [rows, K/32] logical with any strides (MX_SCALE_2D; pass a

@@ -29,6 +29,14 @@ Pinning status (what each function is checked against in ``tests/test_oracle*.py
   * grouped_reference              -> per-expert dense loop (structure of samples/MoE.py:292-334);
                                       the reference holds no test of an MX MoE GEMM:
                                       PARITY UNPINNED beyond the dense per-expert formula.
+  * silu_mul                       -> torch.nn.functional.silu(a) * b (library routine) to a few 1e-7
+                                      relative; closed forms silu(0) = 0, silu(x) -> x for large x,
+                                      silu(-x) -> 0; the reference's own kernel
+                                      (test/kernels/fused_moe.py:85-108) uses approximate division and
+                                      flush-to-zero, so only the formula, not its bits, is the contract
+  * moe_forward                    -> structure of torch_moe (samples/MoE.py:292-334) with the dequantised
+                                      operands; the intermediate re-quantisation is this build's own step:
+                                      PARITY UNPINNED beyond the dense formula (no reference MX MoE exists)
   * bit-level accumulation order of the reference GPU result: PARITY UNPINNED (the arithmetic of
     mma_scaled lives in the closed tileiras compiler and Blackwell hardware).
 """
@@ -328,6 +336,59 @@ def grouped_reference(a_codes, a_scale, w_codes, w_scale, topk_ids, a_fmt=E4M3, 
         w = dequantize(w_codes[e], w_scale[e], w_fmt, block_size)
         out[torch.from_numpy(rows)] = a[torch.from_numpy(rows // topk)] @ w.T
     return out
+
+
+def silu_mul(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """silu(a) * b = a / (1 + exp(-a)) * b (silu_and_mul_kernel, test/kernels/fused_moe.py:85-108) as the
+    fixed sequence of correctly rounded fp32 operations the device executes: exp(-a) = 2^z with
+    z = -a * log2(e) clamped to +-125, z = n + f, n = rint(z), 2^f by the degree-7 Taylor polynomial in
+    f ln 2 evaluated by Horner's rule with separate multiplies and adds, scaled by 2^n exactly."""
+    f32 = np.float32
+    a = np.asarray(a, dtype=f32)
+    b = np.asarray(b, dtype=f32)
+    with np.errstate(invalid="ignore", over="ignore", under="ignore"):
+        z = (-a) * f32(1.44269504)
+        z = np.fmin(np.fmax(z, f32(-125.0)), f32(125.0))
+        n = np.rint(z)
+        f = z - n
+        p = np.full_like(f, f32(1.52527338e-5))
+        for c in (1.54035304e-4, 1.33335581e-3, 9.61812911e-3, 5.55041087e-2, 2.40226507e-1, 6.93147181e-1, 1.0):
+            p = p * f + f32(c)          # numpy rounds the product to fp32 before the add: no fused operation
+        two_n = ((np.nan_to_num(n).astype(np.int32) + 127).astype(np.uint32) << np.uint32(23)).view(f32)
+        e = p * two_n
+        s = f32(1.0) / (f32(1.0) + e)
+        t = np.where(a < f32(-87.5), f32(0.0), a * s)   # exp(-a) is past the clamp: the true value is below 2^-120
+        return t * b
+
+
+def silu_mul_quantize(gate_up: np.ndarray, fmt: str = E4M3, scale_mode: str = "floor"):
+    """silu(gate) * up of a (rows, 2F) array (gate first), MX-quantised along F: the fused producer between
+    the two grouped GEMMs of the MoE pipeline (samples/MoE.py:262-266 followed by block_quantize)."""
+    gate_up = np.asarray(gate_up, dtype=np.float32)
+    F = gate_up.shape[-1] // 2
+    return block_quantize(silu_mul(gate_up[..., :F], gate_up[..., F:]), 32, fmt, scale_mode)
+
+
+def moe_forward(h_codes, h_scale, w1_codes, w1_scale, w2_codes, w2_scale, topk_weights, topk_ids,
+                h_fmt=E4M3, w_fmt=E4M3, scale_mode="floor") -> torch.Tensor:
+    """Block-scaled MoE forward with the structure of cutile_moe / torch_moe (samples/MoE.py:197-334):
+    gate+up projection per routed (token, k) pair, rounded to bf16 as the intermediate buffer is,
+    silu(gate) * up re-quantised to E4M3, down projection, routed-weight multiply, sum over k.
+    Returns fp32 (tokens, H)."""
+    topk_ids = np.asarray(topk_ids)
+    T, topk = topk_ids.shape
+    c1 = grouped_reference(h_codes, h_scale, w1_codes, w1_scale, topk_ids, h_fmt, w_fmt)
+    c1 = c1.to(torch.bfloat16).to(torch.float32).numpy()
+    a2_codes, a2_scale = silu_mul_quantize(c1, E4M3, scale_mode)
+    a2 = dequantize(a2_codes, a2_scale, E4M3)
+    out = torch.zeros((T * topk, w2_codes.shape[1]), dtype=torch.float32)
+    flat = topk_ids.reshape(-1)
+    for e in np.unique(flat):
+        rows = torch.from_numpy(np.nonzero(flat == e)[0])
+        w = dequantize(w2_codes[e], w2_scale[e], w_fmt)
+        out[rows] = a2[rows] @ w.T
+    out = out * torch.as_tensor(np.asarray(topk_weights, dtype=np.float32)).reshape(-1, 1)
+    return out.reshape(T, topk, -1).sum(dim=1)
 
 
 def rel_fro(x: torch.Tensor, ref: torch.Tensor) -> float:

@@ -102,3 +102,35 @@ def test_grouped_gemm_routed_weight_replicas1_and_padded_ids(ct, dev, kernel):
         ct.invoke_fused_moe_scaled(a.storage, a.scale_t, W, ct.pack_scales(Ws), C2, wts.to(dev), sid, eid, True, 1,
                                    256, kernel=kernel)
         assert torch.equal(C, C2)
+
+
+@pytest.mark.parametrize("kernel,tile_m", [("auto", 128), ("auto", 256), ("generic", 16)])
+@pytest.mark.parametrize("w_fmt", [O.E4M3, O.E2M1])
+def test_moe_pipeline_matches_oracle(ct, dev, kernel, tile_m, w_fmt):
+    """cutile_moe_scaled (structure of cutile_moe, samples/MoE.py:197-288) against the oracle's
+    moe_forward.  The intermediate is rounded to bf16 and re-quantised on both sides, so a last-bit
+    difference of the first GEMM can move single elements by one E4M3 step: tolerance 2e-2 relative
+    Frobenius (the reference's own MoE check uses atol 1e-1, samples/MoE.py:462)."""
+    T, H, F, E, topk = 96, 256, 128, 4, 2
+    rng = np.random.default_rng(3)
+    hq, hs = O.block_quantize(rng.standard_normal((T, H)).astype(np.float32), 32, O.E4M3, "floor")
+    w1q, w1s = O.block_quantize((rng.standard_normal((E, 2 * F, H)) * 0.2).astype(np.float32), 32, w_fmt, "floor")
+    w2q, w2s = O.block_quantize((rng.standard_normal((E, H, F)) * 0.2).astype(np.float32), 32, w_fmt, "floor")
+    ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)])
+    wts = rng.random((T, topk)).astype(np.float32)
+    want = O.moe_forward(hq, hs, w1q, w1s, w2q, w2s, wts, ids, w_fmt=w_fmt)
+
+    def dev_elems(codes, fmt):
+        if fmt == O.E2M1:
+            return torch.from_numpy(O.pack_fp4(codes)).to(dev)
+        return torch.from_numpy(codes).to(dev).view(torch.float8_e4m3fn)
+
+    def dev_scale(sc):
+        return torch.from_numpy(sc).to(dev).view(torch.float8_e8m0fnu)
+
+    got = ct.cutile_moe_scaled(dev_elems(hq, O.E4M3), dev_scale(hs), dev_elems(w1q, w_fmt), dev_scale(w1s),
+                               dev_elems(w2q, w_fmt), dev_scale(w2s), torch.from_numpy(wts).to(dev),
+                               torch.from_numpy(ids).to(dev), tile_m, out_dtype=torch.float32,
+                               w_format="e2m1" if w_fmt == O.E2M1 else None, kernel=kernel)
+    assert got.shape == (T, H)
+    assert O.rel_fro(got.cpu(), want) < 2e-2

@@ -162,3 +162,22 @@ def test_pack_scales_layout(ct, dev, rows, KB, form):
             got = ct.pack_scales(big[1:rows + 1, 3:KB + 3]).data.cpu().numpy()
         want = _native_layout(sc)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("in_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("fmt,mode", [(O.E4M3, "floor"), (O.E4M3, "ceil"), (O.E2M1, "floor"), (O.E5M2, "floor")])
+@pytest.mark.parametrize("rows,F", [(5, 32), (33, 96), (16, 48), (7, 1000)])
+def test_silu_mul_quantize_bit_exact(ct, dev, in_dtype, fmt, mode, rows, F):
+    """The fused SiLU(gate) * up + MX quantise pass (silu_and_mul_kernel, test/kernels/fused_moe.py:85-108,
+    then block_quantize) is bit-identical to the oracle's restatement, ragged F and extreme gates included."""
+    g = torch.Generator().manual_seed(rows * 31 + F)
+    x = torch.randn((rows, 2 * F), generator=g) * 4
+    x[0, :8] = torch.tensor([0.0, -0.0, 90.0, -90.0, 1e-30, -200.0, 30.0, -30.0])
+    x = x.to(in_dtype)
+    want_q, want_s = O.silu_mul_quantize(x.float().numpy(), fmt, mode)
+    got_q, got_s = ct.silu_and_mul_quantize(x.to(dev), DT[fmt], scale_mode=mode)
+    got_codes = got_q.view(torch.uint8).cpu().numpy()
+    if fmt == O.E2M1:
+        got_codes = O.unpack_fp4(got_codes)
+    assert np.array_equal(got_s.view(torch.uint8).cpu().numpy(), want_s)
+    assert np.array_equal(got_codes, want_q)

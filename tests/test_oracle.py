@@ -320,3 +320,45 @@ def test_grouped_reference_matches_dense_per_token():
             e = ids[t, j]
             want = O.reference_matmul(a[t:t + 1], sa[t:t + 1], w[e].T.copy(), sw[e].T.copy())
             assert torch.allclose(out[t * topk + j], want[0], rtol=1e-6, atol=1e-6)
+
+
+def test_silu_mul_matches_library_and_closed_forms():
+    """silu_mul (test/kernels/fused_moe.py:85-108) against torch's silu in float64 and its limits."""
+    rng = np.random.default_rng(5)
+    a = (rng.standard_normal(100000) * 8).astype(np.float32)
+    b = rng.standard_normal(100000).astype(np.float32)
+    got = O.silu_mul(a, b).astype(np.float64)
+    ref = (torch.nn.functional.silu(torch.from_numpy(a).double()) * torch.from_numpy(b).double()).numpy()
+    assert np.all(np.abs(got - ref) <= 2e-6 * np.abs(ref) + 1e-37)
+    one = np.ones(5, np.float32)
+    out = O.silu_mul(np.array([0.0, 100.0, -100.0, 1e30, -1e30], np.float32), one)
+    assert out[0] == 0.0 and out[1] == 100.0 and out[2] == 0.0 and out[3] == np.float32(1e30) and out[4] == 0.0
+    assert O.silu_mul(np.array([1.0], np.float32), np.array([2.0], np.float32))[0] == pytest.approx(2 / (1 + np.exp(-1.0)), rel=1e-6)
+    # a dropped minus sign or a swapped operand would show here: silu is not odd and gate comes first
+    assert O.silu_mul(np.array([2.0], np.float32), np.array([0.0], np.float32))[0] == 0.0
+    assert O.silu_mul(np.array([-2.0], np.float32), one[:1])[0] == pytest.approx(-2 / (1 + np.exp(2.0)), rel=1e-6)
+
+
+def test_moe_forward_against_float64_dense_loop():
+    """moe_forward against an independent float64 loop over (token, k) pairs (structure of torch_moe,
+    samples/MoE.py:292-334), with the same intermediate rounding steps applied."""
+    rng = np.random.default_rng(11)
+    T, H, F, E, topk = 6, 64, 32, 3, 2
+    hq, hs = O.block_quantize(rng.standard_normal((T, H)).astype(np.float32), 32, O.E4M3, "floor")
+    w1q, w1s = O.block_quantize((rng.standard_normal((E, 2 * F, H)) * 0.3).astype(np.float32), 32, O.E4M3, "floor")
+    w2q, w2s = O.block_quantize((rng.standard_normal((E, H, F)) * 0.3).astype(np.float32), 32, O.E4M3, "floor")
+    ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)])
+    wts = rng.random((T, topk)).astype(np.float32)
+    got = O.moe_forward(hq, hs, w1q, w1s, w2q, w2s, wts, ids).numpy()
+    h = O.dequantize(hq, hs, O.E4M3).double().numpy()
+    want = np.zeros((T, H))
+    for t in range(T):
+        for j in range(topk):
+            e = ids[t, j]
+            w1 = O.dequantize(w1q[e], w1s[e], O.E4M3).double().numpy()
+            w2 = O.dequantize(w2q[e], w2s[e], O.E4M3).double().numpy()
+            gu = torch.tensor(w1 @ h[t]).float().bfloat16().float().numpy()
+            act = O.silu_mul(gu[:F], gu[F:])
+            aq, asc = O.block_quantize(act[None, :], 32, O.E4M3, "floor")
+            want[t] += wts[t, j] * (w2 @ O.dequantize(aq, asc, O.E4M3).double().numpy()[0])
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-4)
