@@ -340,6 +340,48 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
   return launch_gemm_mfma(g, kernel, (hipStream_t)stream);
 }
 
+namespace {
+// logical (M, N, K) of a problem from its operand descriptors (FP4 operands count elements, not bytes)
+void problem_dims(const mx_tensor& A, const mx_tensor& B, int64_t& M, int64_t& N, int64_t& K) {
+  const int an = A.ndim, bn = B.ndim;
+  M = an >= 2 ? A.shape[an - 2] : 0;
+  K = an >= 2 ? A.shape[an - 1] : 0;
+  N = bn >= 2 ? B.shape[bn - 1] : 0;
+}
+}  // namespace
+
+int64_t mx_gemm_list_workspace_bytes(int32_t count, const mx_tensor* A, const mx_tensor* B,
+                                     const mx_gemm_opts* opts) {
+  if (count <= 0 || !A || !B) return 0;
+  int64_t need = 0;
+  for (int32_t i = 0; i < count; ++i) {
+    int64_t M, N, K;
+    problem_dims(A[i], B[i], M, N, K);
+    const int64_t b = mx_gemm_workspace_bytes(M, N, K, opts);
+    need = b > need ? b : need;
+  }
+  return need;
+}
+
+int mx_gemm_list(int32_t count, const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const mx_tensor* Bs,
+                 mx_tensor* C, const mx_gemm_opts* opts, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (count < 0) return set_error(MX_ERR_INVALID, "mx_gemm_list: negative count");
+  if (count == 0) return MX_OK;
+  if (!A || !As || !B || !Bs || !C) return set_error(MX_ERR_INVALID, "mx_gemm_list: null descriptor array");
+  for (int32_t i = 0; i < count; ++i) {
+    int64_t M, N, K;
+    problem_dims(A[i], B[i], M, N, K);
+    if (A[i].ndim == 2 && B[i].ndim == 2 && (M == 0 || N == 0)) continue;
+    const int rc = mx_gemm(&A[i], &As[i], &B[i], &Bs[i], &C[i], opts, workspace, workspace_bytes, stream);
+    if (rc != MX_OK) {
+      char inner[400];
+      snprintf(inner, sizeof inner, "%s", mx_last_error());
+      return set_error(rc, "problem %d of the list: %s", (int)i, inner);
+    }
+  }
+  return MX_OK;
+}
+
 int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W, const mx_tensor* Ws,
                     mx_tensor* C, const float* topk_weights, const int32_t* sorted_token_ids,
                     int64_t num_slots, const int32_t* sorted_expert_ids, int32_t tile_m,

@@ -238,6 +238,67 @@ def block_scaled_matmul(A: torch.Tensor, A_scale, B: torch.Tensor, B_scale, *,
                         kernel=kernel, block=32)
 
 
+def grouped_block_scaled_matmul(As, A_scales, Bs, B_scales, *, out_dtype: torch.dtype = torch.float32,
+                                Cs=None, kernel: str = "auto"):
+    """A list of independent block-scaled products ``Cs[i] = (As[i] * A_scales[i]) @ (Bs[i] * B_scales[i])``
+    whose sizes may all differ: the block-scaled counterpart of the reference's list-of-problems
+    ``grouped_matmul_kernel(As, Bs, Cs, ...)`` (test/kernels/group_gemm.py:10-38, driven as in
+    test/test_group_gemm.py).  Every problem follows the rules of :func:`block_scaled_matmul`; all are
+    enqueued by one library call on the current stream.  Returns the list of outputs."""
+    n = len(As)
+    if not (len(A_scales) == len(Bs) == len(B_scales) == n) or (Cs is not None and len(Cs) != n):
+        raise ValueError("As, A_scales, Bs, B_scales (and Cs) must be lists of the same length")
+    if n == 0:
+        return []
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise TileTypeError(f"Unsupported output dtype {_dtype_name(out_dtype)}, expected float32 or bfloat16")
+    dA, dAs, dB, dBs, dC = ((L.MxTensor * n)() for _ in range(5))
+    outs, keep, layouts = [], [], set()
+    dev = As[0].device
+    for i in range(n):
+        A, B = As[i], Bs[i]
+        a_fmt, b_fmt = _elem_format(A, None), _elem_format(B, None)
+        if a_fmt is None or b_fmt is None:
+            bad = A if a_fmt is None else B
+            raise TileTypeError(f"Unsupported input dtype {_dtype_name(bad.dtype)} for mma_scaled, supported "
+                                "input dtypes are float8_e4m3fn, float8_e5m2, float4_e2m1fn")
+        if A.dim() != 2 or B.dim() != 2:
+            raise TileTypeError(f"Expect A and B to be 2D, got {tuple(A.shape)} and {tuple(B.shape)}")
+        a_pd = _packed_dim(A, 1, None) if a_fmt == "e2m1" else -1
+        b_pd = _packed_dim(B, 0, None) if b_fmt == "e2m1" else -1
+        a_log, b_log = _logical_shape(A, a_pd), _logical_shape(B, b_pd)
+        if a_log[1] != b_log[0]:
+            raise ValueError(f"Incompatible matrices: K dimension of A ({a_log[1]}) "
+                             f"must match K dimension of B ({b_log[0]})")
+        if not A.is_cuda or A.device != dev or B.device != dev:
+            raise ValueError("Input tensors must be on the same CUDA device.")
+        M, K, N = a_log[0], a_log[1], b_log[1]
+        C = torch.empty((M, N), device=dev, dtype=out_dtype) if Cs is None else Cs[i]
+        if tuple(C.shape) != (M, N) or C.dtype not in (torch.float32, torch.bfloat16) or C.device != dev:
+            raise ValueError(f"C must be a ({M}, {N}) float32 or bfloat16 tensor on {dev}")
+        au, bu = _as_u8(A), _as_u8(B)
+        keep += [au, bu]
+        dA[i] = L.desc(au, _FMT_CODE[a_fmt], a_pd)
+        dB[i] = L.desc(bu, _FMT_CODE[b_fmt], b_pd)
+        dAs[i], la = _scale_desc(A_scales[i], M, K, 32, False)
+        dBs[i], lb = _scale_desc(B_scales[i], N, K, 32, True)
+        layouts.add((la, lb))
+        dC[i] = L.desc(C, L._TORCH_TO_MX[C.dtype])
+        outs.append(C)
+    if len(layouts) != 1:
+        raise TileValueError("all problems of a list must pass their scales in the same layout")
+    la, lb = layouts.pop()
+    o = _opts(False, la, lb, kernel, 32)
+    lib = L.lib()
+    need = lib.mx_gemm_list_workspace_bytes(n, dA, dB, ctypes.byref(o))
+    ws = _workspace(dev, need)
+    with torch.cuda.device(dev):
+        rc = lib.mx_gemm_list(n, dA, dAs, dB, dBs, dC, ctypes.byref(o), ws.data_ptr() if ws is not None else None,
+                              need, L.stream_ptr(dev))
+    _check(rc)
+    return outs
+
+
 def cutile_block_scaled_matmul(A, A_scale, B, B_scale) -> torch.Tensor:
     """Exact signature of the reference sample wrapper (fp32 result)."""
     return block_scaled_matmul(A, A_scale, B, B_scale)

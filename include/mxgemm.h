@@ -140,6 +140,21 @@ MX_API int mx_gemm(const mx_tensor* A, const mx_tensor* A_scale, const mx_tensor
             int64_t workspace_bytes, void* stream);
 
 /*
+ * A list of independent block-scaled products C[i] = A[i] x B[i] (problem sizes may all differ), the
+ * block-scaled counterpart of grouped_matmul_kernel(As, Bs, Cs, ...), test/kernels/group_gemm.py:10-38.
+ * The descriptor arrays hold `count` entries each; every problem follows the rules of mx_gemm and is
+ * enqueued on `stream` in list order (no host synchronisation; one workspace of
+ * mx_gemm_list_workspace_bytes, the largest single need, is reused from problem to problem, which stream
+ * order makes safe).  Empty problems (M or N zero) are skipped.  On error the index of the failing
+ * problem is part of mx_last_error() and nothing after it is enqueued.
+ */
+MX_API int64_t mx_gemm_list_workspace_bytes(int32_t count, const mx_tensor* A, const mx_tensor* B,
+                                     const mx_gemm_opts* opts);
+MX_API int mx_gemm_list(int32_t count, const mx_tensor* A, const mx_tensor* A_scale, const mx_tensor* B,
+                 const mx_tensor* B_scale, mx_tensor* C, const mx_gemm_opts* opts, void* workspace,
+                 int64_t workspace_bytes, void* stream);
+
+/*
  * Grouped (MoE) variant.  Replaces: ct.launch(..., fused_moe_kernel, (A, B, C, topk_weights,
  * sorted_token_ids, sorted_expert_ids, num_token_replicas, mul_routed_weight, TILE_M, TILE_N,
  * TILE_K)) -- samples/MoE.py:338-375, kernel test/kernels/fused_moe.py:14-82, with the bf16 ct.mma

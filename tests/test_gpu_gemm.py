@@ -151,3 +151,34 @@ def test_concurrent_launch_threads(ct, dev):
     [t.start() for t in ts]
     [t.join() for t in ts]
     assert not errs, errs
+
+
+@pytest.mark.parametrize("kernel", ["auto", "generic", "mfma128"])
+def test_list_of_problems(ct, dev, kernel):
+    """The list API (block-scaled counterpart of grouped_matmul_kernel, test/kernels/group_gemm.py:10-38;
+    the reference's test, test/test_group_gemm.py, also mixes problem sizes): every problem of a list with
+    different sizes and element formats matches its own oracle product; an empty problem is skipped."""
+    shapes = [(128, 256, 512, O.E4M3, O.E4M3), (33, 80, 96, O.E4M3, O.E2M1), (300, 130, 2048, O.E2M1, O.E2M1),
+              (0, 64, 64, O.E4M3, O.E4M3), (512, 512, 1024, O.E5M2, O.E5M2)]
+    ops = [(randn_operand(m, k, fa, 900 + i, dev), randn_operand(n, k, fb, 950 + i, dev))
+           for i, (m, n, k, fa, fb) in enumerate(shapes)]
+    got = ct.grouped_block_scaled_matmul([a.storage if a.fmt != O.E2M1 else a.storage.view(torch.float4_e2m1fn_x2)
+                                          for a, _ in ops],
+                                         [a.scale_t for a, _ in ops],
+                                         [(b.storage if b.fmt != O.E2M1 else b.storage.view(torch.float4_e2m1fn_x2)).T
+                                          for _, b in ops],
+                                         [b.scale_t.T for _, b in ops], kernel=kernel)
+    assert len(got) == len(shapes)
+    for (a, b), c, (m, n, k, _, _) in zip(ops, got, shapes):
+        assert tuple(c.shape) == (m, n)
+        if m:
+            _check(c, oracle_matmul(a, b), torch.float32, f"list {m}x{n}x{k}")
+
+
+def test_list_of_problems_reports_the_failing_index(ct, dev):
+    a = randn_operand(64, 64, O.E4M3, 1, dev)
+    b = randn_operand(64, 64, O.E4M3, 2, dev)
+    bad_scale = torch.zeros((64, 3), dtype=torch.uint8, device=dev).view(torch.float8_e8m0fnu)
+    with pytest.raises(Exception, match="problem 1 of the list"):
+        ct.grouped_block_scaled_matmul([a.storage, a.storage], [a.scale_t, bad_scale],
+                                       [b.storage.T, b.storage.T], [b.scale_t.T, b.scale_t.T])
