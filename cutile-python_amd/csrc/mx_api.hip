@@ -218,6 +218,30 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
   }
   if (M == 0 || N == 0) return MX_OK;
 
+  // ---- batched operands (test/test_mma_scaled.py:128-145): one 2-D product per batch entry, size-1
+  // batches broadcast; stream order lets the entries share the workspace.  Layouts only the generic
+  // kernel reads (block 16, E4M3 scales) keep its own batched launch. --------------------------------
+  if (batched && o.kernel != MX_KERNEL_GENERIC && o.block_size == 32 && As->dtype == MX_E8M0 &&
+      o.a_scale_layout == MX_SCALE_2D && o.b_scale_layout == MX_SCALE_2D) {
+    auto slice = [](const mx_tensor* t, int64_t b, int elem_bytes) {
+      mx_tensor v = *t;
+      if (t->ndim == 3) {
+        v.ptr = (uint8_t*)t->ptr + (t->shape[0] > 1 ? b : 0) * t->stride[0] * elem_bytes;
+        v.ndim = 2;
+        for (int i = 0; i < 2; ++i) { v.shape[i] = t->shape[i + 1]; v.stride[i] = t->stride[i + 1]; }
+        if (v.packed_dim >= 0) v.packed_dim -= 1;
+      }
+      return v;
+    };
+    const int c_bytes = C->dtype == MX_BF16 ? 2 : 4;
+    for (int64_t b = 0; b < batch; ++b) {
+      const mx_tensor a2 = slice(A, b, 1), as2 = slice(As, b, 1), b2 = slice(B, b, 1), bs2 = slice(Bs, b, 1);
+      mx_tensor c2 = slice(C, b, c_bytes);
+      if (int rc = mx_gemm(&a2, &as2, &b2, &bs2, &c2, &o, workspace, workspace_bytes, stream)) return rc;
+    }
+    return MX_OK;
+  }
+
   // ---- can the MFMA path take it? ------------------------------------------------------------------
   const char* why = nullptr;
   const int64_t a_ld = A->stride[and_ - 2], b_ld = B->stride[bnd - 1];

@@ -69,6 +69,24 @@ def test_batch_mma_scaled_fp8(ct, dev):
     torch.testing.assert_close(out.cpu(), ref, atol=1e-2, rtol=1e-2)
 
 
+def test_batch_mma_scaled_k_contiguous_broadcast(ct, dev):
+    """Batched operands whose matrices are K-contiguous (y given as the transposed view of (b, n, k)) take
+    the MFMA kernels entry by entry; x has a batch of one and is broadcast (test/test_mma_scaled.py:128-145,
+    batch rules src/cuda/tile/_stub.py:2232-2235)."""
+    b, m, n, k, ks = 3, 96, 160, 256, 8
+    g = torch.Generator().manual_seed(21)
+    X = torch.randn((1, m, k), generator=g).to(torch.float8_e4m3fn)
+    Yt = torch.randn((b, n, k), generator=g).to(torch.float8_e4m3fn)
+    Xs, Yst = _scales((1, m, ks), 22), _scales((b, n, ks), 23)
+    Z = torch.randn((b, m, n), generator=g)
+    ref = _ref(X.view(torch.uint8).numpy(), Xs.view(torch.uint8).numpy(),
+               Yt.view(torch.uint8).numpy().transpose(0, 2, 1), Yst.view(torch.uint8).numpy().transpose(0, 2, 1),
+               Z, O.E4M3, 32)
+    out = ct.mma_scaled(X.to(dev), Xs.to(dev), Yt.to(dev).transpose(1, 2), Yst.to(dev).transpose(1, 2), Z.to(dev))
+    assert out.shape == (b, m, n)
+    assert O.rel_fro(out.cpu(), ref) < 1e-3
+
+
 @pytest.mark.parametrize("scale_dtype,block", [(f8e8m0, 32), (f8e8m0, 16), (torch.float8_e4m3fn, 16)], ids=str)
 def test_mma_scaled_general_f4(ct, dev, scale_dtype, block):
     m, n, k = 16, 16, 64
