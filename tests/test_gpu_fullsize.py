@@ -1,0 +1,104 @@
+"""GPU parity at the full sizes of the benchmark configurations, through properties that do not need a
+full CPU product: exact scaling by powers of two, bit-identical results from two independent kernels,
+the checksum identity C 1 = A (B 1) evaluated in float64, and sampled rows against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _operand(ct, dev, rows, K, fmt, seed, std=1.0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    x = torch.randn((rows, K), generator=g, device=dev) * std
+    q, s = ct.block_quantize(x, 32, torch.float8_e4m3fn if fmt == O.E4M3 else "e2m1", scale_mode="floor")
+    return q, s
+
+
+def _dequant_cpu(q, s, fmt):
+    codes = q.view(torch.uint8).cpu().numpy()
+    if fmt == O.E2M1:
+        codes = O.unpack_fp4(codes)
+    return O.dequantize(codes, s.view(torch.uint8).cpu().numpy(), fmt)
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E2M1])
+def test_square_8192_properties(ct, dev, fmt):
+    """MXFP8 / MXFP4 8192^3, bf16 output (the headline configurations)."""
+    M = N = K = 8192
+    kw = {} if fmt == O.E4M3 else {"a_format": "e2m1", "b_format": "e2m1"}
+    a_q, a_s = _operand(ct, dev, M, K, fmt, 101)
+    b_q, b_s = _operand(ct, dev, N, K, fmt, 102)
+    c = ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, out_dtype=torch.bfloat16, **kw)
+
+    # two independent kernels (persistent ping-pong, one-tile-per-workgroup) accumulate every output in the
+    # same K order: bit-identical
+    c_ref = ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, out_dtype=torch.bfloat16, kernel="mfma256", **kw)
+    assert torch.equal(c.view(torch.int16), c_ref.view(torch.int16))
+
+    # doubling every A scale (E8M0 byte + 1) doubles the result exactly
+    a_s2 = (a_s.view(torch.uint8) + 1).view(torch.float8_e8m0fnu)
+    c2 = ct.block_scaled_matmul(a_q, a_s2, b_q.T, b_s.T, out_dtype=torch.bfloat16, **kw)
+    assert torch.equal(c2.float(), 2.0 * c.float())
+
+    # checksum of checksums over all 64 Mi outputs: C 1 = A (B 1) in float64
+    a = _dequant_cpu(a_q, a_s, fmt).double()
+    b = _dequant_cpu(b_q, b_s, fmt).double()
+    want = a @ b.sum(dim=0)
+    got = c.double().sum(dim=1).cpu()
+    # bf16 rounding: 2^-9 relative per output, independent over the 8192 outputs of a row
+    row_norm = torch.sqrt(((a * a) @ (b * b).sum(dim=0)))     # ~ l2 norm of the row of C
+    assert bool(((got - want).abs() <= 6 * 2.0 ** -9 * row_norm + 1e-6).all())
+
+    # sampled rows against the oracle, every column
+    rows = torch.from_numpy(np.random.default_rng(7).choice(M, 64, replace=False))
+    ref = a[rows].float() @ b.float().T
+    assert O.rel_fro(c[rows.to(dev)].float().cpu(), ref) < 8e-3
+
+
+def test_decode_shape_properties(ct, dev):
+    """M = 32 activations (E4M3) x 28672 x 8192 FP4 weights, bf16 output."""
+    M, N, K = 32, 28672, 8192
+    x_q, x_s = _operand(ct, dev, M, K, O.E4M3, 201)
+    w_q, w_s = _operand(ct, dev, N, K, O.E2M1, 202, std=0.02)
+    c = ct.block_scaled_matmul(x_q, x_s, w_q.T, w_s.T, out_dtype=torch.bfloat16, b_format="e2m1")
+    c_tiled = ct.block_scaled_matmul(x_q, x_s, w_q.T, w_s.T, out_dtype=torch.bfloat16, b_format="e2m1",
+                                     kernel="mfma128")
+    # the decode kernel splits K over 8 waves and sums the partials: not the tiled kernel's order, so the
+    # comparison is by tolerance; both against the oracle
+    x = _dequant_cpu(x_q, x_s, O.E4M3)
+    w = _dequant_cpu(w_q, w_s, O.E2M1)
+    ref = x @ w.T
+    assert O.rel_fro(c.float().cpu(), ref) < 8e-3
+    assert O.rel_fro(c_tiled.float().cpu(), ref) < 8e-3
+    x_s2 = (x_s.view(torch.uint8) + 2).view(torch.float8_e8m0fnu)
+    c4 = ct.block_scaled_matmul(x_q, x_s2, w_q.T, w_s.T, out_dtype=torch.bfloat16, b_format="e2m1")
+    assert torch.equal(c4.float(), 4.0 * c.float())
+
+
+def test_moe_shape_properties(ct, dev):
+    """MoE up-projection of the benchmark: 4096 tokens, H = 4096, 8 experts, F = 14336, top-2."""
+    T, H, E, F, topk, tile_m = 4096, 4096, 8, 14336, 2, 256
+    a_q, a_s = _operand(ct, dev, T, H, O.E4M3, 301)
+    w_q, w_s = _operand(ct, dev, E * F, H, O.E4M3, 302, std=0.05)
+    w_q, w_s = w_q.view(E, F, H), w_s.view(E, F, H // 32)
+    g = torch.Generator().manual_seed(303)
+    ids = torch.topk(torch.rand((T, E), generator=g), topk, dim=1).indices
+    sid, eid = ct.moe_align_tile_size(ids.to(dev), tile_m, E, exact=False)
+    c = torch.zeros((T, topk, F), dtype=torch.bfloat16, device=dev)
+    ct.invoke_fused_moe_scaled(a_q, a_s, w_q, w_s, c, None, sid, eid, False, topk, tile_m)
+    c_ref = torch.zeros_like(c)
+    ct.invoke_fused_moe_scaled(a_q, a_s, w_q, w_s, c_ref, None, sid, eid, False, topk, tile_m, kernel="mfma128")
+    assert torch.equal(c.view(torch.int16), c_ref.view(torch.int16))
+    # sampled (token, k) pairs against the dense per-expert formula
+    a = _dequant_cpu(a_q, a_s, O.E4M3)
+    rng = np.random.default_rng(9)
+    for e in range(E):
+        pairs = np.argwhere(ids.numpy() == e)
+        pick = pairs[rng.choice(len(pairs), min(8, len(pairs)), replace=False)]
+        w = _dequant_cpu(w_q[e], w_s[e], O.E4M3)
+        ref = a[pick[:, 0]] @ w.T
+        got = c[torch.from_numpy(pick[:, 0]).to(dev), torch.from_numpy(pick[:, 1]).to(dev)].float().cpu()
+        assert O.rel_fro(got, ref) < 8e-3
