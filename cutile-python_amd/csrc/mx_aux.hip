@@ -8,9 +8,11 @@ namespace {
 // ================================================================================================
 // MX quantiser (replaces the torch-op chain of block_quantize, test/kernels/kernel_utils.py:38-80)
 // ================================================================================================
-// Element conversion is done on the bit pattern: value = sig * 2^(ex-150) is divided by the block
-// scale 2^se by subtracting exponents, then rounded to nearest even onto the target grid in one step.
-// No floating-point operation is involved, so denormal modes and fused operations cannot change a bit.
+// The shared exponent is computed on bit patterns.  Element conversion has two routes with identical
+// results: the gfx950 scaled-conversion instructions for ordinary blocks, and an integer route (value =
+// sig * 2^(ex-150) divided by 2^se by subtracting exponents, then rounded to nearest even onto the target
+// grid in one step) for blocks with a zero / subnormal amax, inf / NaN or an extreme scale, where denormal
+// modes or the instruction's special cases could otherwise change a bit.
 
 struct Unpacked {
   uint32_t sig;   // 24-bit significand with the leading one at bit 23 (0 for zero)
@@ -128,29 +130,51 @@ __device__ inline void load4_as_f32(const void* p, int64_t i, int dtype, bool ve
   }
 }
 
-// 8 lanes per 32-element block, 4 consecutive elements per lane.
-__global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
-  const int64_t KB = q.Kpad / 32;
-  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t blk = gid >> 3;
-  const int sub = (int)(gid & 7);
-  const bool live = blk < q.rows * KB;
-  const int64_t row = live ? blk / KB : 0, kb = live ? blk % KB : 0;
-  const int64_t k0 = kb * 32 + sub * 4;
+// Where unit `gid` (8 consecutive units = one 32-element block, 4 consecutive elements per unit) lives.
+struct QuantUnit {
+  int64_t row, kb, k0;
+  int sub;
+  bool live;
+};
 
-  float v[4] = {0.f, 0.f, 0.f, 0.f};
-  if (live) {
-    const int64_t base = row * q.x_ld + k0;
-    const int esz = q.x_dtype == MX_F32 ? 4 : 2;
+__device__ inline QuantUnit quant_unit(const QuantArgs& q, int64_t gid) {
+  const int64_t KB = q.Kpad / 32;
+  QuantUnit u;
+  const int64_t blk = gid >> 3;
+  u.sub = (int)(gid & 7);
+  u.live = blk < q.rows * KB;
+  if (q.rows * KB < ((int64_t)1 << 31)) {   // uniform: 32-bit division is several times cheaper
+    const uint32_t b32 = u.live ? (uint32_t)blk : 0u, kb32 = (uint32_t)KB;
+    u.row = b32 / kb32;
+    u.kb = b32 - (uint32_t)u.row * kb32;
+  } else {
+    u.row = u.live ? blk / KB : 0;
+    u.kb = u.live ? blk % KB : 0;
+  }
+  u.k0 = u.kb * 32 + u.sub * 4;
+  return u;
+}
+
+// the (at most) four input values of a unit; the fused producer applies silu(x) * up
+__device__ inline void quant_load(const QuantArgs& q, const QuantUnit& u, float* v, float* w) {
+  for (int e = 0; e < 4; ++e) v[e] = w[e] = 0.f;
+  if (!u.live) return;
+  const int64_t base = u.row * q.x_ld + u.k0;
+  const int esz = q.x_dtype == MX_F32 ? 4 : 2;
+  const int nvalid = q.K - u.k0 >= 4 ? 4 : (q.K > u.k0 ? (int)(q.K - u.k0) : 0);
+  const bool vec = nvalid == 4 && q.x_dtype != MX_F16 &&
+                   ((((uintptr_t)q.x) | ((uintptr_t)q.up) | (uintptr_t)(q.x_ld * esz)) & (4 * esz - 1)) == 0;
+  load4_as_f32(q.x, base, q.x_dtype, vec, nvalid, v);
+  if (q.up) load4_as_f32(q.up, base, q.x_dtype, vec, nvalid, w);
+}
+
+__device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float* v, const float* w) {
+  const bool live = u.live;
+  const int64_t row = u.row, kb = u.kb, k0 = u.k0;
+  const int sub = u.sub;
+  if (q.up) {
     const int nvalid = q.K - k0 >= 4 ? 4 : (q.K > k0 ? (int)(q.K - k0) : 0);
-    const bool vec = nvalid == 4 && q.x_dtype != MX_F16 &&
-                     ((((uintptr_t)q.x) | ((uintptr_t)q.up) | (uintptr_t)(q.x_ld * esz)) & (4 * esz - 1)) == 0;
-    load4_as_f32(q.x, base, q.x_dtype, vec, nvalid, v);
-    if (q.up) {
-      float u[4];
-      load4_as_f32(q.up, base, q.x_dtype, vec, nvalid, u);
-      for (int e = 0; e < 4; ++e) v[e] = e < nvalid ? silu_mul_f32(v[e], u[e]) : 0.f;
-    }
+    for (int e = 0; e < 4; ++e) v[e] = (live && e < nvalid) ? silu_mul_f32(v[e], w[e]) : 0.f;
   }
   // amax over the block on |bits| (monotone in |x| for finite values; NaN patterns compare largest)
   uint32_t bits[4], am = 0;
@@ -187,11 +211,44 @@ __global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
   const bool saturate = q.scale_mode != 0;
 
   uint32_t code[4];
-  for (int e = 0; e < 4; ++e) {
-    const Unpacked u = unpack_f32(bits[e]);
-    code[e] = q.fmt == MX_E4M3 ? encode_e4m3(u, se, saturate)
-              : q.fmt == MX_E5M2 ? encode_e5m2(u, se, saturate)
-                                 : encode_e2m1(u, se);
+  // Blocks whose amax is a normal finite number and whose scale 2^se is a normal float take the hardware
+  // scaled conversions (v_cvt_scalef32_pk_*: x / 2^se rounded to nearest even; FP8 overflows to NaN / inf,
+  // FP4 saturates -- measured on MI355X against the integer encoders below for 270 k inputs per format).
+  // The saturating FP8 rule clamps the magnitude to max_normal * 2^se first, which is exact.  Everything
+  // else (zero or subnormal amax, inf / NaN, extreme scales) goes through the integer encoders.
+  if (am >= 0x00800000u && am < 0x7F800000u && se > -127 && se < 120) {
+    typedef short s2 __attribute__((ext_vector_type(2)));
+    const float sc = __builtin_bit_cast(float, (uint32_t)(se + 127) << 23);
+    float x[4];
+    for (int e = 0; e < 4; ++e) x[e] = v[e];
+    if (saturate && q.fmt != MX_E2M1) {
+      const float lim = __fmul_rn(q.fmt == MX_E4M3 ? 448.0f : 57344.0f, sc);
+      for (int e = 0; e < 4; ++e) x[e] = __builtin_copysignf(fminf(__builtin_fabsf(x[e]), lim), x[e]);
+    }
+    uint32_t packed;
+    if (q.fmt == MX_E4M3) {
+      s2 r = {0, 0};
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(r, x[0], x[1], sc, false);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(r, x[2], x[3], sc, true);
+      packed = __builtin_bit_cast(uint32_t, r);
+    } else if (q.fmt == MX_E5M2) {
+      s2 r = {0, 0};
+      r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(r, x[0], x[1], sc, false);
+      r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(r, x[2], x[3], sc, true);
+      packed = __builtin_bit_cast(uint32_t, r);
+    } else {
+      uint32_t r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, x[0], x[1], sc, 0);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, x[2], x[3], sc, 1);
+      packed = (r & 0xFu) | ((r & 0xF0u) << 4) | ((r & 0xF00u) << 8) | ((r & 0xF000u) << 12);
+    }
+    for (int e = 0; e < 4; ++e) code[e] = (packed >> (8 * e)) & 0xFFu;
+  } else {
+    for (int e = 0; e < 4; ++e) {
+      const Unpacked u = unpack_f32(bits[e]);
+      code[e] = q.fmt == MX_E4M3 ? encode_e4m3(u, se, saturate)
+                : q.fmt == MX_E5M2 ? encode_e5m2(u, se, saturate)
+                                   : encode_e2m1(u, se);
+    }
   }
   if (!live) return;
   if (q.fmt == MX_E2M1) {
@@ -208,6 +265,23 @@ __global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
     }
   }
   if (sub == 0) q.scale[row * q.sc_ld + kb] = (uint8_t)(se + 127);
+}
+
+// 8 lanes per 32-element block, 4 consecutive elements per lane; every thread handles kQuantUnroll units a
+// grid apart and requests all their inputs before it processes the first (memory-level parallelism).
+constexpr int kQuantUnroll = 1;
+__global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
+  const int64_t nthreads = (int64_t)gridDim.x * 256;
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  QuantUnit u[kQuantUnroll];
+  float v[kQuantUnroll][4], w[kQuantUnroll][4];
+#pragma unroll
+  for (int i = 0; i < kQuantUnroll; ++i) {
+    u[i] = quant_unit(q, gid + i * nthreads);
+    quant_load(q, u[i], v[i], w[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < kQuantUnroll; ++i) quant_store(q, u[i], v[i], w[i]);
 }
 
 // ================================================================================================
@@ -434,9 +508,9 @@ __global__ __launch_bounds__(256) void moe_align_seg_kernel(const int32_t* __res
 }  // namespace
 
 int launch_quantize(const QuantArgs& q, hipStream_t stream) {
-  const int64_t threads = q.rows * (q.Kpad / 32) * 8;
-  if (threads <= 0) return MX_OK;
-  const int64_t blocks = (threads + 255) / 256;
+  const int64_t units = q.rows * (q.Kpad / 32) * 8;
+  if (units <= 0) return MX_OK;
+  const int64_t blocks = (units + 256 * kQuantUnroll - 1) / (256 * kQuantUnroll);
   if (blocks > 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "quantize: tensor too large");
   hipLaunchKernelGGL(quantize_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, q);
   hipError_t e = hipGetLastError();

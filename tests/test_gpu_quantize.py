@@ -181,3 +181,30 @@ def test_silu_mul_quantize_bit_exact(ct, dev, in_dtype, fmt, mode, rows, F):
         got_codes = O.unpack_fp4(got_codes)
     assert np.array_equal(got_s.view(torch.uint8).cpu().numpy(), want_s)
     assert np.array_equal(got_codes, want_q)
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2, O.E2M1])
+@pytest.mark.parametrize("mode", ["floor", "ceil"])
+def test_quantize_dense_rounding_grid(ct, dev, fmt, mode):
+    """Every block holds one anchor (which fixes the shared exponent) and 31 values from a dense grid of
+    fractions of it: all rounding ties, the subnormal range of the element format, values just below and
+    above the largest finite code.  Bit-exact against the oracle (encoders pinned by tests/test_oracle.py)."""
+    rng = np.random.default_rng(17)
+    anchors = np.array([1.0, 1.75, 447.9, 448.0, 3.0e-5, 7.3e11, 0.013, 5.99, 6.0, 57344.0], np.float32)
+    fr = np.concatenate([np.arange(0, 4097, dtype=np.float64) / 4096.0,             # 12-bit fractions: all ties
+                         2.0 ** -np.arange(1, 24, dtype=np.float64) * 1.5,           # deep into the subnormals
+                         1.0 + np.arange(-8, 9, dtype=np.float64) * 2.0 ** -10])     # around the anchor itself
+    fr = fr[: (len(fr) // 31) * 31].reshape(-1, 31)
+    blocks = []
+    for a in anchors:
+        for row in fr:
+            sign = rng.choice([-1.0, 1.0], 31)
+            blocks.append(np.concatenate([[a], np.minimum(row, 1.0) * a * sign]))
+    x = np.asarray(blocks, np.float32).reshape(-1, 32 * 7)                            # 7 blocks per row
+    want_q, want_s = O.block_quantize(x, 32, fmt, mode)
+    got_q, got_s = ct.block_quantize(torch.from_numpy(x).to(dev), 32, DT[fmt], scale_mode=mode)
+    got_codes = got_q.view(torch.uint8).cpu().numpy()
+    if fmt == O.E2M1:
+        got_codes = O.unpack_fp4(got_codes)
+    assert np.array_equal(got_s.view(torch.uint8).cpu().numpy(), want_s)
+    assert np.array_equal(got_codes, want_q)
