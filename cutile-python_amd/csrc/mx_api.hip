@@ -30,7 +30,29 @@ int big_tile_kernel() {
   return pp ? MX_KERNEL_MFMA_PINGPONG : MX_KERNEL_MFMA_256x256;
 }
 
-const mx_gemm_opts kDefaultOpts = {sizeof(mx_gemm_opts), 0, MX_SCALE_2D, MX_SCALE_2D, MX_KERNEL_AUTO, 32, {0, 0}};
+const mx_gemm_opts kDefaultOpts = {sizeof(mx_gemm_opts), 0, MX_SCALE_2D, MX_SCALE_2D, MX_KERNEL_AUTO, 32, 0, 0};
+
+// Number of K-slices for a problem that ends up on a one-tile MFMA kernel (1 = no split).  Depends only on
+// (M, N, K, opts) so that mx_gemm_workspace_bytes and mx_gemm agree.  Automatic rule: split when the tiles
+// of the 128x128 kernel cover less than half of the CUs and every slice keeps at least two K-quads.
+int plan_k_splits(int64_t M, int64_t N, int64_t K, const mx_gemm_opts& o) {
+  if (o.split_k == 1 || o.a_scale_layout != MX_SCALE_2D || o.b_scale_layout != MX_SCALE_2D || o.block_size != 32)
+    return 1;
+  if (o.kernel != MX_KERNEL_AUTO && o.kernel != MX_KERNEL_MFMA_128x128 && o.kernel != MX_KERNEL_MFMA_256x256 &&
+      o.kernel != MX_KERNEL_MFMA_256x256_W4)
+    return 1;
+  if (K <= 0 || K % 512 != 0 || M <= 0 || N <= 0) return 1;
+  if (o.split_k > 1) return (K % ((int64_t)512 * o.split_k) == 0) ? o.split_k : -1;   // -1: cannot honour
+  if (o.kernel != MX_KERNEL_AUTO && o.kernel != MX_KERNEL_MFMA_128x128) return 1;
+  if (o.kernel == MX_KERNEL_AUTO && M > 128 && N > 128 && M * N >= (int64_t)1024 * 1024) return 1;   // big-tile kernel
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  if (tiles * 2 > 256 || K < 2048) return 1;
+  int64_t s = 256 / tiles;
+  if (s > K / 1024) s = K / 1024;
+  while (s > 1 && K % (512 * s) != 0) --s;
+  return (int)(s < 1 ? 1 : s);
+}
+
 
 int check_tensor(const mx_tensor* t, const char* name, int min_nd, int max_nd) {
   if (!t) return set_error(MX_ERR_INVALID, "%s: null descriptor", name);
@@ -94,6 +116,12 @@ int64_t mx_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, const mx_gemm_o
   const mx_gemm_opts& o = opts ? *opts : kDefaultOpts;
   if (o.kernel == MX_KERNEL_GENERIC) return 0;
   int64_t b = 0;
+  const int S = plan_k_splits(M, N, K, o);
+  if (S > 1) {   // per-slice packed scales and the fp32 partial products
+    b += S * (mx_packed_scale_bytes(M, K / S) + mx_packed_scale_bytes(N, K / S));
+    b += round256(S * M * N * 4);
+    return b;
+  }
   if (o.a_scale_layout != MX_SCALE_NATIVE) b += mx_packed_scale_bytes(M, K);
   if (o.b_scale_layout != MX_SCALE_NATIVE) b += mx_packed_scale_bytes(N, K);
   return b;
@@ -268,6 +296,10 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
     return set_error(MX_ERR_LAYOUT, "requested kernel %d cannot run this problem: %s", kernel, why);
   }
 
+  if (o.split_k > 1 && kernel != MX_KERNEL_MFMA_128x128 && kernel != MX_KERNEL_MFMA_256x256 &&
+      kernel != MX_KERNEL_MFMA_256x256_W4)
+    return set_error(MX_ERR_LAYOUT, "split_k = %d is only available on the one-tile MFMA kernels (kernel %d chosen)",
+                     o.split_k, kernel);
   if (kernel == MX_KERNEL_GENERIC) {
     if (o.a_scale_layout == MX_SCALE_NATIVE || o.b_scale_layout == MX_SCALE_NATIVE)
       return set_error(MX_ERR_LAYOUT, "the generic kernel cannot read native-layout scales");
@@ -334,6 +366,43 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
   const uint32_t* as_native = (const uint32_t*)As->ptr;
   const uint32_t* bs_native = (const uint32_t*)Bs->ptr;
   PackArgs pa, pb;
+  int S = 1;
+  if (kernel == MX_KERNEL_MFMA_128x128 || kernel == MX_KERNEL_MFMA_256x256 || kernel == MX_KERNEL_MFMA_256x256_W4) {
+    S = plan_k_splits(M, N, K, o);
+    if (S < 0)
+      return set_error(MX_ERR_SHAPE, "split_k = %d needs K (%lld) to be a multiple of %d", o.split_k, (long long)K,
+                       512 * o.split_k);
+  }
+  if (S > 1) {
+    // ---- split-K: the slices are a batch for the scale re-layout and a second grid dimension for the GEMM
+    const int64_t Ks = K / S, kbs = Ks / 32;
+    if (int rc = make_pack_args(As, MX_SCALE_2D, M, K, ws, pa)) return rc;
+    pa.K = Ks; pa.batch = S; pa.s_batch = kbs * pa.s_kb;
+    const uint32_t* as_p = (const uint32_t*)ws;
+    ws += S * mx_packed_scale_bytes(M, Ks);
+    mx_tensor t = *Bs;   // [K/32, N] -> view as [N, K/32]
+    t.shape[0] = Bs->shape[1]; t.shape[1] = Bs->shape[0];
+    t.stride[0] = Bs->stride[1]; t.stride[1] = Bs->stride[0];
+    if (int rc = make_pack_args(&t, MX_SCALE_2D, N, K, ws, pb)) return rc;
+    pb.K = Ks; pb.batch = S; pb.s_batch = kbs * pb.s_kb;
+    const uint32_t* bs_p = (const uint32_t*)ws;
+    ws += S * mx_packed_scale_bytes(N, Ks);
+    float* partial = (float*)ws;
+    if (int rc = launch_pack_scales_pair(&pa, &pb, (hipStream_t)stream)) return rc;
+    GemmArgs g = {};
+    g.A = (const uint8_t*)A->ptr; g.B = (const uint8_t*)B->ptr; g.As = as_p; g.Bs = bs_p; g.C = partial;
+    g.lda = a_ld; g.ldb = b_ld; g.ldc = N;
+    g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)Ks;
+    g.a_fmt = A->dtype; g.b_fmt = B->dtype; g.c_dtype = MX_F32; g.accumulate = 0;
+    g.a_rows = M;
+    g.replicas = 1;
+    g.k_splits = S;
+    g.as_split_stride = mx_packed_scale_bytes(M, Ks) / 4;
+    g.bs_split_stride = mx_packed_scale_bytes(N, Ks) / 4;
+    g.c_split_stride = M * N;
+    if (int rc = launch_gemm_mfma(g, kernel, (hipStream_t)stream)) return rc;
+    return launch_splitk_reduce(partial, S, M, N, C->ptr, C->stride[0], C->dtype, o.accumulate, (hipStream_t)stream);
+  }
   const bool pack_a = o.a_scale_layout != MX_SCALE_NATIVE, pack_b = o.b_scale_layout != MX_SCALE_NATIVE;
   if (pack_a) {
     if (int rc = make_pack_args(As, o.a_scale_layout, M, K, ws, pa)) return rc;

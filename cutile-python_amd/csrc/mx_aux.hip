@@ -505,6 +505,37 @@ __global__ __launch_bounds__(256) void moe_align_seg_kernel(const int32_t* __res
   for (int64_t blk = used / tile_m + tid; blk < max_slots / tile_m; blk += T) expert_ids[blk] = 0;
 }
 
+// ================================================================================================
+// Split-K reduction: C = sum of the fp32 partial products (analogue of the second pass of
+// matmul_split_k_kernel, test/kernels/matmul.py:103-140)
+// ================================================================================================
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int splits,
+                                                            int64_t M, int64_t N, void* C, int64_t ldc,
+                                                            int c_dtype, int accumulate) {
+  const int64_t n4 = (N + 3) / 4;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= M * n4) return;
+  const int64_t m = i / n4, n = (i % n4) * 4;
+  const int cnt = N - n >= 4 ? 4 : (int)(N - n);
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int p = 0; p < splits; ++p) {   // fixed order: results do not depend on scheduling
+    const float* src = part + ((int64_t)p * M + m) * N + n;
+    if (cnt == 4 && (N & 3) == 0) {
+      const v4f t = *(const v4f*)src;
+      s[0] += t.x; s[1] += t.y; s[2] += t.z; s[3] += t.w;
+    } else {
+      for (int e = 0; e < cnt; ++e) s[e] += src[e];
+    }
+  }
+  if (c_dtype == MX_F32) {
+    float* c = (float*)C + m * ldc + n;
+    for (int e = 0; e < cnt; ++e) c[e] = accumulate ? c[e] + s[e] : s[e];
+  } else {
+    uint16_t* c = (uint16_t*)C + m * ldc + n;
+    for (int e = 0; e < cnt; ++e) c[e] = f32_to_bf16(accumulate ? bf16_to_f32(c[e]) + s[e] : s[e]);
+  }
+}
+
 }  // namespace
 
 int launch_quantize(const QuantArgs& q, hipStream_t stream) {
@@ -542,6 +573,17 @@ int launch_pack_scales_pair(const PackArgs* a, const PackArgs* b, hipStream_t st
 
 int launch_pack_scales(const PackArgs& p, hipStream_t stream) {
   return launch_pack_scales_pair(&p, nullptr, stream);
+}
+
+int launch_splitk_reduce(const float* partials, int splits, int64_t M, int64_t N, void* C, int64_t ldc,
+                         int c_dtype, int accumulate, hipStream_t stream) {
+  const int64_t threads = M * ((N + 3) / 4);
+  if (threads <= 0) return MX_OK;
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, partials,
+                     splits, M, N, C, ldc, c_dtype, accumulate);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "splitk_reduce_kernel launch: %s", hipGetErrorString(e));
+  return MX_OK;
 }
 
 int launch_moe_align(const int32_t* topk_ids, int64_t num_ids, int32_t num_experts, int32_t tile_m,

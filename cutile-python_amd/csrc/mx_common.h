@@ -95,10 +95,18 @@ struct GemmArgs {
   int64_t bs_expert_stride;  // dwords between experts in Bs
   int64_t a_rows;            // rows of the A tensor (for the buffer descriptor)
   int32_t stagger;           // 1: workgroups start their K walk at different quads
+  // split-K (one-tile kernels only): K is the slice length, slice i reads the scales / writes the partial
+  // output i strides further on
+  int32_t k_splits;
+  int64_t as_split_stride, bs_split_stride;   // dwords
+  int64_t c_split_stride;                     // elements of C
 };
 
 int launch_gemm_mfma(const GemmArgs& g, int kernel_id, hipStream_t stream);
 int launch_gemm_pingpong(const GemmArgs& g, hipStream_t stream);
+// C[m, n] (+)= sum over `splits` fp32 partials [splits][M][N]; C fp32 or bf16 with row pitch ldc
+int launch_splitk_reduce(const float* partials, int splits, int64_t M, int64_t N, void* C, int64_t ldc,
+                         int c_dtype, int accumulate, hipStream_t stream);
 
 struct GenericArgs {
   const uint8_t* A; const uint8_t* As; const uint8_t* B; const uint8_t* Bs; void* C;

@@ -64,7 +64,12 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
   }
   const int m0 = tile_m * C::BM, n0 = tile_n * C::BN;
 
-  const int Kb_a = g.K * C::A_EB / 8, Kb_b = g.K * C::B_EB / 8;   // bytes per row
+  // Split-K: blockIdx.y owns the K range [split * g.K, (split + 1) * g.K) of the full problem (g.K is the
+  // slice length, a whole number of K-quads), its own slice of the packed scales and its own fp32 partial
+  // output; a reduction kernel adds the partials.
+  const int split = blockIdx.y;
+  const int ka0 = split * (g.K * C::A_EB / 8), kb0 = split * (g.K * C::B_EB / 8);   // first byte of the slice
+  const int Kb_a = ka0 + g.K * C::A_EB / 8, Kb_b = kb0 + g.K * C::B_EB / 8;         // end of the slice in a row
   const int ksteps = (g.K + 127) / 128;
   const int nstages = (ksteps + C::KSUB - 1) / C::KSUB;
   const int KQ = (ksteps + 3) / 4;
@@ -114,13 +119,13 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
   auto issue_one = [&](int idx, int s, int buf, bool live) {
     lds_u8* const abase = smem + buf * C::STAGE;
     if (idx < C::A_LOADS) {
-      const int q = idx, ka = s * C::A_RB;
+      const int q = idx, ka = ka0 + s * C::A_RB;
       uint32_t v = a_voff[q];
       if (!live || ka + a_col[q] >= Kb_a) v = kOobOffset;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_void*)(abase + (q * C::NW + wave) * 1024), 16, v,
                                                ka, 0, 0);
     } else {
-      const int q = idx - C::A_LOADS, kb = s * C::B_RB;
+      const int q = idx - C::A_LOADS, kb = kb0 + s * C::B_RB;
       uint32_t v = b_voff[q];
       if (!live || kb + b_col[q] >= Kb_b) v = kOobOffset;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(abase + C::A_STAGE + (q * C::NW + wave) * 1024),
@@ -132,8 +137,9 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
   constexpr int AQ = C::MT / 4, BQ = C::NTL / 4;
   // the packed tensors hold ceil(rows / 64) row groups; a tile that hangs over the matrix edge re-reads
   // the last group (its rows are never stored)
-  const v4i* const as_ptr = (const v4i*)g.As + lane;
-  const v4i* const bs_ptr = (const v4i*)(g.Bs + (GROUPED ? (int64_t)expert * g.bs_expert_stride : 0)) + lane;
+  const v4i* const as_ptr = (const v4i*)(g.As + (int64_t)split * g.as_split_stride) + lane;
+  const v4i* const bs_ptr = (const v4i*)(g.Bs + (GROUPED ? (int64_t)expert * g.bs_expert_stride : 0) +
+                                         (int64_t)split * g.bs_split_stride) + lane;
   const int a_groups = (g.M + 63) / 64, b_groups = (g.N + 63) / 64;
   int a_grp[AQ], b_grp[BQ];
 #pragma unroll
@@ -242,8 +248,8 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
   }
 
   // ---- epilogue: lane (r, gq) of tile (i, j) holds C[m0+wm0+16i+r][n0+wn0+16j+4gq .. +3] -----------
-  OutT* const Cp = (OutT*)g.C;
-  const bool vec_ok = (g.ldc % 4 == 0) && (((uintptr_t)g.C) % 16 == 0);
+  OutT* const Cp = (OutT*)g.C + (int64_t)split * g.c_split_stride;
+  const bool vec_ok = (g.ldc % 4 == 0) && (((uintptr_t)g.C) % 16 == 0) && (g.c_split_stride % 4 == 0);
   const bool accumulate = g.accumulate != 0;
 #pragma unroll
   for (int i = 0; i < C::MT; ++i) {
@@ -283,7 +289,8 @@ int launch_one(const GemmArgs& g, hipStream_t stream) {
   }
   const int64_t tiles = (int64_t)((g.M + C::BM - 1) / C::BM) * ((g.N + C::BN - 1) / C::BN);
   if (tiles <= 0) return MX_OK;
-  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(C::NT), C::LDS_BYTES, stream, g);
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)(g.k_splits > 1 ? g.k_splits : 1)), dim3(C::NT),
+                     C::LDS_BYTES, stream, g);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "gemm_kernel launch: %s", hipGetErrorString(e));
   return MX_OK;

@@ -41,7 +41,7 @@ class MxGemmOpts(ctypes.Structure):
     _fields_ = [("struct_size", ctypes.c_int32), ("accumulate", ctypes.c_int32),
                 ("a_scale_layout", ctypes.c_int32), ("b_scale_layout", ctypes.c_int32),
                 ("kernel", ctypes.c_int32), ("block_size", ctypes.c_int32),
-                ("reserved", ctypes.c_int32 * 2)]
+                ("split_k", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
 
 # every symbol include/mxgemm.h declares: name -> (restype, argtypes)

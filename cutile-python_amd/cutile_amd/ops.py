@@ -110,7 +110,7 @@ def _as_u8(t: torch.Tensor) -> torch.Tensor:
     return t if t.dtype == torch.uint8 else t.view(torch.uint8)
 
 
-def _opts(accumulate=False, a_layout=L.MX_SCALE_2D, b_layout=L.MX_SCALE_2D, kernel="auto", block=32):
+def _opts(accumulate=False, a_layout=L.MX_SCALE_2D, b_layout=L.MX_SCALE_2D, kernel="auto", block=32, split_k=0):
     o = L.MxGemmOpts()
     o.struct_size = ctypes.sizeof(L.MxGemmOpts)
     o.accumulate = int(bool(accumulate))
@@ -120,6 +120,7 @@ def _opts(accumulate=False, a_layout=L.MX_SCALE_2D, b_layout=L.MX_SCALE_2D, kern
         raise TileValueError(f"unknown kernel {kernel!r}; expected one of {sorted(L.KERNELS)}")
     o.kernel = L.KERNELS[kernel]
     o.block_size = block
+    o.split_k = int(split_k)
     return o
 
 
@@ -159,7 +160,7 @@ def _workspace(dev: torch.device, nbytes: int) -> Optional[torch.Tensor]:
     return buf
 
 
-def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kernel, block):
+def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kernel, block, split_k=0):
     dev = A.device
     and_, bnd = A.dim(), B.dim()
     a_log = _logical_shape(A, a_pd if a_fmt == "e2m1" else -1)
@@ -170,7 +171,7 @@ def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kerne
     dAs, la = _scale_desc(As, M, K, block, False)
     dBs, lb = _scale_desc(Bs, N, K, block, True)
     dC = L.desc(C, L._TORCH_TO_MX[C.dtype])
-    o = _opts(accumulate, la, lb, kernel, block)
+    o = _opts(accumulate, la, lb, kernel, block, split_k)
     lib = L.lib()
     need = lib.mx_gemm_workspace_bytes(M, N, K, ctypes.byref(o))
     ws = _workspace(dev, need)
@@ -188,7 +189,7 @@ def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kerne
 def block_scaled_matmul(A: torch.Tensor, A_scale, B: torch.Tensor, B_scale, *,
                         out_dtype: torch.dtype = torch.float32, C: Optional[torch.Tensor] = None,
                         accumulate: bool = False, a_format: Optional[str] = None,
-                        b_format: Optional[str] = None, kernel: str = "auto") -> torch.Tensor:
+                        b_format: Optional[str] = None, kernel: str = "auto", split_k: int = 0) -> torch.Tensor:
     """C = (A * A_scale) @ (B * B_scale) with fp32 accumulation, returned as ``out_dtype``.
 
     A (M, K) and B (K, N) hold MX elements: ``float8_e4m3fn`` / ``float8_e5m2``, or FP4 E2M1 packed two
@@ -198,7 +199,8 @@ def block_scaled_matmul(A: torch.Tensor, A_scale, B: torch.Tensor, B_scale, *,
     :class:`PackedScales`.  The two operands may use different element formats (for example E4M3
     activations with E2M1 weights): the hardware takes them independently.  The fast kernels need
     K-contiguous operands, i.e. B given as the transposed view of an (N, K) tensor as the reference
-    sample does; other layouts run on a slower general kernel.
+    sample does; other layouts run on a slower general kernel.  ``split_k``: 0 lets the library split a
+    long K over several workgroups when M x N alone cannot fill the GPU, 1 forbids it, n > 1 forces n slices.
     """
     a_fmt, b_fmt = _elem_format(A, a_format), _elem_format(B, b_format)
     if a_fmt is None or b_fmt is None:
@@ -235,7 +237,7 @@ def block_scaled_matmul(A: torch.Tensor, A_scale, B: torch.Tensor, B_scale, *,
         if tuple(C.shape) != (m, n) or C.dtype not in (torch.float32, torch.bfloat16) or C.device != A.device:
             raise ValueError(f"C must be a ({m}, {n}) float32 or bfloat16 tensor on {A.device}")
     return _launch_gemm(A, a_fmt, a_pd, A_scale, B, b_fmt, b_pd, B_scale, C, accumulate=accumulate,
-                        kernel=kernel, block=32)
+                        kernel=kernel, block=32, split_k=split_k)
 
 
 def grouped_block_scaled_matmul(As, A_scales, Bs, B_scales, *, out_dtype: torch.dtype = torch.float32,

@@ -102,7 +102,13 @@ typedef struct mx_gemm_opts {
   int32_t b_scale_layout;
   int32_t kernel;         /* MX_KERNEL_*                                                         */
   int32_t block_size;     /* scaling block size B along K: 32 (16 only with MX_KERNEL_GENERIC)   */
-  int32_t reserved[2];
+  int32_t split_k;        /* mx_gemm only: 0 = the library decides, 1 = never split K, n > 1 = n K-slices
+                             (K must be a multiple of 512 n; plain 2-D scale layouts; one-tile MFMA
+                             kernels).  Slices run side by side and a second kernel adds their fp32
+                             partial products in a fixed order: the split-K scheme of
+                             matmul_split_k_kernel, test/kernels/matmul.py:103-140, for small M x N
+                             with a long K                                                        */
+  int32_t reserved;
 } mx_gemm_opts;
 
 /* Library version (MXGEMM_VERSION of the built library). */

@@ -182,3 +182,30 @@ def test_list_of_problems_reports_the_failing_index(ct, dev):
     with pytest.raises(Exception, match="problem 1 of the list"):
         ct.grouped_block_scaled_matmul([a.storage, a.storage], [a.scale_t, bad_scale],
                                        [b.storage.T, b.storage.T], [b.scale_t.T, b.scale_t.T])
+
+
+@pytest.mark.parametrize("M,N,K,split_k", [(64, 256, 8192, 0), (200, 130, 4096, 4), (128, 128, 16384, 0),
+                                           (96, 512, 2048, 2), (33, 64, 1024, 2)])
+@pytest.mark.parametrize("fa,fb,out_dtype", [(O.E4M3, O.E4M3, torch.float32), (O.E4M3, O.E2M1, torch.bfloat16)])
+def test_split_k(ct, dev, M, N, K, split_k, fa, fb, out_dtype):
+    """Small M x N with a long K: slices of K run side by side and a second kernel adds the fp32 partials
+    (the scheme of matmul_split_k_kernel, test/kernels/matmul.py:103-140).  Automatic (0) and forced splits,
+    ragged M / N, with and without accumulation into C; M > 32 keeps the mixed-format case off the decode kernel."""
+    a, b = randn_operand(M, K, fa, 700 + M, dev), randn_operand(N, K, fb, 800 + N, dev)
+    ref = oracle_matmul(a, b)
+    c = _run(ct, a, b, out_dtype=out_dtype, split_k=split_k)
+    _check(c, ref, out_dtype, f"split_k={split_k} {M}x{N}x{K}")
+    c1 = _run(ct, a, b, out_dtype=out_dtype, split_k=1)
+    _check(c1, ref, out_dtype, "unsplit")
+    z = torch.randn((M, N), generator=torch.Generator().manual_seed(5)).to(out_dtype)
+    acc = z.to(dev).clone()
+    _run(ct, a, b, C=acc, accumulate=True, split_k=split_k)
+    _check(acc, ref + z.float(), out_dtype, "split-K accumulate")
+
+
+def test_split_k_rejects_impossible_requests(ct, dev):
+    a, b = randn_operand(64, 1536, O.E4M3, 1, dev), randn_operand(64, 1536, O.E4M3, 2, dev)
+    with pytest.raises(Exception, match="multiple of"):
+        _run(ct, a, b, split_k=2)          # 1536 is not a multiple of 1024
+    with pytest.raises(Exception, match="one-tile MFMA kernels"):
+        _run(ct, a, b, split_k=3, kernel="generic")
