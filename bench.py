@@ -161,6 +161,23 @@ def bench_gemm(ct, O, dev, M, N, K, fmt, dist, steps, warmup, check, nsets=3):
             "kernel_tflops": flops / t_kernel * 1e-12, "rel_fro_vs_oracle": err, "flops": flops, "sets": sets}
 
 
+def vendor_scaled_mm(sets, steps, warmup):
+    """Context only, not part of the product path: the vendor library's MXFP8 GEMM (torch._scaled_mm with
+    E8M0 scales, hipBLASLt underneath) on the same operands, timed like the kernel-only leg."""
+    def run(i):
+        a_q, a_s, b_q, b_s, _ = sets[i % len(sets)]
+        return torch._scaled_mm(a_q, b_q.T, scale_a=a_s, scale_b=b_s, out_dtype=torch.bfloat16)
+    try:
+        run(0)
+        _sync()
+        t = _time_events(run, steps, warmup)
+    except Exception as e:   # an image without MX support in its BLAS: report that, the bench goes on
+        return {"error": f"{type(e).__name__}: {str(e)[:160]}"}
+    M, K = sets[0][0].shape
+    N = sets[0][2].shape[0]
+    return {"kernel_ms": t * 1e3, "tflops": 2.0 * M * N * K / t * 1e-12}
+
+
 def bench_decode(ct, O, dev, steps, warmup, check, nsets=8):
     """Decode-shaped mixed GEMM: X MXFP8 (32, 8192) x W MXFP4 (28672, 8192)^T, bf16 out.  HBM bound; the
     121 MiB working set fits in the Infinity Cache, so 8 weight sets are rotated."""
@@ -291,6 +308,8 @@ def main():
     ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c5 (default: all)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the correctness check before timing")
+    ap.add_argument("--no-vendor", action="store_true",
+                    help="skip the context leg that times torch._scaled_mm on the headline operands")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (a known-size reference for "
                          "scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -353,6 +372,8 @@ def main():
                          "kernel": "gemm_pp_kernel<Cfg<e4m3,e4m3,256,256,2,4>,bf16>", "kernel_ms": r["kernel_ms"],
                          "flops_per_launch": r["flops"]},
         })
+        if not a.no_vendor:
+            extra["context_torch_scaled_mm_mxfp8_8192"] = vendor_scaled_mm(r["sets"], a.steps, a.warmup)
         if not a.no_cpu:
             out["cpu_baseline"] = cpu_baseline_c2(O, r["sets"])
     else:

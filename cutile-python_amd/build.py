@@ -23,6 +23,10 @@ SOURCES = ["mx_api.hip", "mx_gemm_mfma.hip", "mx_gemm_pp.hip", "mx_gemm_generic.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          f"-I{INCLUDE}", f"-I{CSRC}", "-Wno-unused-command-line-argument"]
+# Kernel variants with parts of the work removed (for timing studies; their results are invalid) are only
+# compiled into a library built with MXGEMM_TIMING_AIDS=1 in the environment -- never the shipped one.
+if os.environ.get("MXGEMM_TIMING_AIDS") == "1":
+    FLAGS.append("-DMXGEMM_TIMING_AIDS")
 
 
 def _newer(src: pathlib.Path, obj: pathlib.Path) -> bool:

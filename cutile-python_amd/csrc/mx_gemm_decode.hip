@@ -259,6 +259,9 @@ template <int XF, int SPW, int MT, typename OutT>
 int launch_decode_k(const DecodeArgs& d, int grid, hipStream_t stream) {
   using Cf = DecodeCfg<SPW, MT>;
   auto kern = decode_kernel<XF, SPW, MT, OutT>;
+#ifdef MXGEMM_TIMING_AIDS
+  // Only in builds made with -DMXGEMM_TIMING_AIDS (never the shipped library): MXGEMM_DEC selects a variant
+  // with parts of the work removed (results invalid): 1 no MFMA / LDS reads, 2 no reduction, 4 no X loads
   static const int var = [] { const char* e = getenv("MXGEMM_DEC"); return e ? atoi(e) : 0; }();
   if constexpr (SPW == 8 && MT == 2 && sizeof(OutT) == 2) {
     if (var == 1) kern = decode_kernel<XF, SPW, MT, OutT, 1>;
@@ -268,6 +271,7 @@ int launch_decode_k(const DecodeArgs& d, int grid, hipStream_t stream) {
     if (var == 7) kern = decode_kernel<XF, SPW, MT, OutT, 7>;
     if (var != 0) hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);
   }
+#endif
   static int attr_done = 0;   // benign race: the attribute call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);

@@ -211,6 +211,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   OutT* const Cp = (OutT*)g.C;
   const bool vec_ok = (g.ldc % 4 == 0) && (((uintptr_t)g.C) % 16 == 0);
   const bool accumulate = g.accumulate != 0;
+  int eid[2] = {-1, -1};
   auto write_tile = [&](int m0, int n0) {
     if constexpr (!GROUPED) {
       // interior tile, plain store: one address per lane, everything else immediate offsets
@@ -239,27 +240,47 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
         write_tile_checked<OutT>(t, Cp, g.ldc, g.M, g.N, m0 + wm0 + r, n0 + wn0 + 4 * gq, accumulate, vec_ok);
       return;
     }
+    // grouped: row 16 i + c of the team's half goes to row `id` of C, where id is the routed-slot index
+    // that lane 16 (i % 4) + c of eid[i / 4] has held since the tile began (no load latency here)
+    const bool cols_in = n0 + 256 <= g.N && vec_ok && !accumulate;   // uniform
+    float ewt[2] = {1.f, 1.f};
+    if (g.topk_weights) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+        if (eid[u] >= 0 && eid[u] < g.num_valid_ids) ewt[u] = g.topk_weights[eid[u]];
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int m = m0 + wm0 + 16 * i + r;
-      int64_t orow = m;
-      bool ok = m < g.M;
+      const int src = (16 * (i & 3) + r) * 4;
+      const int id = __builtin_amdgcn_ds_bpermute(src, eid[i >> 2]);
+      const bool ok = id >= 0 && id < g.num_valid_ids;
       float w = 1.f;
-      if constexpr (GROUPED) {
-        const int id = ok ? g.sorted_token_ids[m] : 0x7FFFFFFF;
-        ok = ok && id >= 0 && id < g.num_valid_ids;
-        orow = id;
-        if (ok && g.topk_weights) w = g.topk_weights[id];
+      if (g.topk_weights) w = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, ewt[i >> 2])));
+      OutT* const p = Cp + (int64_t)id * g.ldc + (n0 + wn0 + 4 * gq);
+      if (cols_in) {
+        if ((!(VAR & 2) || g.ldc == -12345) && ok) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) store4_full<OutT>(p + 16 * j, acc[i][j] * w);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int n = n0 + wn0 + 16 * j + 4 * gq;
+          if ((!(VAR & 2) || g.ldc == -12345) && ok && n < g.N)
+            store4<OutT>(p + 16 * j, acc[i][j] * w, accumulate, g.N - n, vec_ok);
+        }
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int n = n0 + wn0 + 16 * j + 4 * gq;
-        if ((!(VAR & 2) || g.ldc == -12345) && ok && n < g.N) {
-          v4f v = acc[i][j];
-          if constexpr (GROUPED) v *= w;
-          store4<OutT>(Cp + orow * g.ldc + n, v, accumulate, g.N - n, vec_ok);
-        }
-        acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  // grouped: the routed-slot ids of the team's 128 rows of the tile at m0, two per lane
+  auto load_row_ids = [&](int m0) {
+    if constexpr (GROUPED) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int m = m0 + wm0 + 64 * u + lane;
+        eid[u] = m < g.M ? g.sorted_token_ids[m] : -1;
       }
     }
   };
@@ -267,6 +288,11 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   // ---- prologue: stages 0 and 1 of the first tile, scales of its K-quad 0 ---------------------------------
   int lid = walk.first;          // tile being computed
   set_fetch_tile(lid);
+  {
+    int fm0, fn0;
+    walk.origin(lid, fm0, fn0);
+    load_row_ids(fm0);
+  }
   issue_a(0, 0);
   issue_b(0, 0);
   issue_a(1, 1);
@@ -293,6 +319,10 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
         int pm0, pn0;
         walk.origin(lid - walk.step, pm0, pn0);
         write_tile(pm0, pn0);
+        if constexpr (GROUPED) {
+          walk.origin(lid, pm0, pn0);
+          load_row_ids(pm0);
+        }
       }
     }
     // from stage nstages - 2 on, the loads run ahead into the next tile of the walk
@@ -480,21 +510,36 @@ int launch_gemm_pingpong(const GemmArgs& g, hipStream_t stream) {
   if (g.c_dtype != MX_F32 && g.c_dtype != MX_BF16)
     return set_error(MX_ERR_DTYPE, "MFMA kernel: output dtype %d not supported", g.c_dtype);
   const bool grouped = g.sorted_token_ids != nullptr;
-  // timing aids (MXGEMM_PP_VAR, read once): 1 no DMA in the loop, 2 no output stores, 4 no late LDS reads
+#ifdef MXGEMM_TIMING_AIDS
+  // Only in builds made with -DMXGEMM_TIMING_AIDS (never the shipped library): MXGEMM_PP_VAR, read once,
+  // selects a variant with parts of the work removed (results invalid): 1 no DMA in the loop, 2 no output
+  // stores, 4 no late LDS reads, 8 DMA of cache-resident data
   static const int var_env = [] { const char* e = getenv("MXGEMM_PP_VAR"); return e ? (int)strtol(e, nullptr, 0) : 0; }();
-  if (var_env && g.a_fmt == MX_E4M3 && g.b_fmt == MX_E4M3 && g.c_dtype == MX_BF16 && !grouped) {
+  if (var_env && g.a_fmt == MX_E4M3 && g.b_fmt == MX_E4M3 && g.c_dtype == MX_BF16) {
     using C = Cfg<MX_E4M3, MX_E4M3, 256, 256, 2, 4>;
-    switch (var_env) {
-      case 1: return launch_pp<C, uint16_t, false, 1>(g, stream);
-      case 2: return launch_pp<C, uint16_t, false, 2>(g, stream);
-      case 3: return launch_pp<C, uint16_t, false, 3>(g, stream);
-      case 4: return launch_pp<C, uint16_t, false, 4>(g, stream);
-      case 5: return launch_pp<C, uint16_t, false, 5>(g, stream);
-      case 7: return launch_pp<C, uint16_t, false, 7>(g, stream);
-      case 8: return launch_pp<C, uint16_t, false, 8>(g, stream);
-      case 10: return launch_pp<C, uint16_t, false, 10>(g, stream);
+    if (grouped) {
+      switch (var_env) {
+        case 1: return launch_pp<C, uint16_t, true, 1>(g, stream);
+        case 2: return launch_pp<C, uint16_t, true, 2>(g, stream);
+        case 4: return launch_pp<C, uint16_t, true, 4>(g, stream);
+        case 5: return launch_pp<C, uint16_t, true, 5>(g, stream);
+        case 7: return launch_pp<C, uint16_t, true, 7>(g, stream);
+        case 8: return launch_pp<C, uint16_t, true, 8>(g, stream);
+      }
+    } else {
+      switch (var_env) {
+        case 1: return launch_pp<C, uint16_t, false, 1>(g, stream);
+        case 2: return launch_pp<C, uint16_t, false, 2>(g, stream);
+        case 3: return launch_pp<C, uint16_t, false, 3>(g, stream);
+        case 4: return launch_pp<C, uint16_t, false, 4>(g, stream);
+        case 5: return launch_pp<C, uint16_t, false, 5>(g, stream);
+        case 7: return launch_pp<C, uint16_t, false, 7>(g, stream);
+        case 8: return launch_pp<C, uint16_t, false, 8>(g, stream);
+        case 10: return launch_pp<C, uint16_t, false, 10>(g, stream);
+      }
     }
   }
+#endif
 #define MX_CASE(AFMT, BFMT)                                                                        \
   if (g.a_fmt == AFMT && g.b_fmt == BFMT) {                                                        \
     using C = Cfg<AFMT, BFMT, 256, 256, 2, 4>;                                                     \
