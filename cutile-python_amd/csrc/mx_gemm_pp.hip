@@ -98,9 +98,10 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
                                         const int lane, const TileWalk& walk) {
   using P = PP<C>;
   constexpr int AL = P::AL, BL = P::BL;
-  // A tiles (of 8) whose fragments are read in the memory phase; the gather / scatter bookkeeping of the
-  // grouped variant leaves registers for two only
-  constexpr int EARLY = GROUPED ? 2 : 4;
+  // A tiles (of 8) whose fragments are read in the memory phase; the others are read inside the MFMA phase,
+  // 8 MFMAs ahead of their use.  Two measured best (four: 1.5 % slower on MXFP8, 5 % on the grouped
+  // variant: the longer memory phase costs more than the later reads)
+  constexpr int EARLY = 2;
   const int r = lane & 15, gq = lane >> 4;
   constexpr int wm0 = TEAM * 128;
   const int wn0 = wn * 64;
