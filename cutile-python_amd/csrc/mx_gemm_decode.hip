@@ -255,6 +255,236 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
 #undef MX_ISSUE_TILE
 }
 
+// ---- variant for 16 < M <= 32 with K = 4 * SPW * 128 ---------------------------------------------------
+// The 8 waves are 4 K-slices x 2 halves of M (16 rows of X each), so a K-slice is twice as long as in
+// decode_kernel and, at K = 8192, one DMA instruction reads 1 KiB of ONE weight row instead of 512 bytes of
+// two (HBM streams long contiguous pieces measurably faster).  The two waves of a K-slice multiply the same
+// weight fragments by their own half of X, so a tile is shared through LDS: each of the two loads half of
+// the slice's rows, one workgroup barrier tells that a tile has landed and one that its slot may be
+// refilled.  LDS slot of a tile: [K-slice][row][slice bytes] (16-byte chunks XOR-swizzled by row), then
+// [row][K/32] scale bytes; two slots, i.e. two tiles in flight per workgroup.
+template <int SPW>
+struct Decode2Cfg {
+  static constexpr int SLB = SPW * 64;            // bytes of a weight row inside one K-slice
+  static constexpr int LPR = SLB / 16;            // lanes (16-byte chunks) per row of a slice
+  static constexpr int RPI = 64 / LPR;            // rows per DMA instruction
+  static constexpr int WIW = 16 / RPI / 2;        // weight DMA instructions per wave and tile
+  static constexpr int SROW = SPW * 16;           // scale bytes per weight row (K / 32)
+  static constexpr int LS = SROW / 16;            // lanes per scale row
+  static constexpr int S_INSTR = 16 * SROW / 1024;   // scale DMA instructions per tile (waves 0 .. S_INSTR-1)
+  static constexpr int W_BYTES = 4 * 16 * SLB;
+  static constexpr int SLOT = W_BYTES + 16 * SROW;
+  static constexpr int RING = 2 * SLOT;
+  static constexpr int RED = kWaves * kBatch * 64 * 16;
+  static constexpr int LDS_BYTES = RING > RED ? RING : RED;
+};
+
+template <int SPW>
+__device__ inline void issue_tile_dma2(const uint8_t* W, uint32_t wbytes, const uint8_t* S, uint32_t sbytes,
+                                       lds_u8* wdst, lds_u8* sdst, const uint32_t* woff, uint32_t soff,
+                                       int wsoff, int ssoff, bool with_scales) {
+  using Cf = Decode2Cfg<SPW>;
+  const __amdgpu_buffer_rsrc_t rsW = make_rsrc(W, wbytes), rsS = make_rsrc(S, sbytes);
+#pragma unroll
+  for (int j = 0; j < Cf::WIW; ++j)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsW, (lds_void*)(wdst + j * 1024), 16, woff[j], wsoff, 0, 0);
+  if (with_scales)   // uniform per wave
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsS, (lds_void*)sdst, 16, soff, ssoff, 0, 0);
+}
+
+template <int XF, int SPW, typename OutT>
+__global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d) {
+  using Cf = Decode2Cfg<SPW>;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
+  lds_u8* const smem = (lds_u8*)smem_generic;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int q = wave & 3, mh = wave >> 2;      // K-slice, half of M
+  const int r = lane & 15, gq = lane >> 4;
+  const bool with_scales = wave < Cf::S_INSTR;
+
+  // ---- per-lane DMA offsets inside a tile --------------------------------------------------------------
+  const uint32_t wbytes = (uint32_t)((int64_t)d.N * d.ldw), sbytes = (uint32_t)((int64_t)d.N * d.ldws);
+  uint32_t woff[Cf::WIW];
+#pragma unroll
+  for (int j = 0; j < Cf::WIW; ++j) {
+    const int rr = (mh * Cf::WIW + j) * Cf::RPI + lane / Cf::LPR, p = lane % Cf::LPR;
+    const int c = p ^ (rr & 15);               // chunk of the row that lives at LDS position p
+    woff[j] = (uint32_t)(rr * d.ldw + q * Cf::SLB + c * 16);
+  }
+  const uint32_t soff = (uint32_t)((wave * (64 / Cf::LS) + lane / Cf::LS) * d.ldws + (lane % Cf::LS) * 16);
+  auto issue = [&](int tile, int slot) {
+    lds_u8* const base = smem + slot * Cf::SLOT;
+    issue_tile_dma2<SPW>(d.W, wbytes, d.Ws, sbytes, base + q * (16 * Cf::SLB) + mh * Cf::WIW * 1024,
+                         base + Cf::W_BYTES + wave * 1024, woff, soff, tile * 16 * (int)d.ldw,
+                         tile * 16 * (int)d.ldws, with_scales);
+  };
+
+  // tiles of this workgroup: blockIdx.x, + gridDim.x, ... -- at any moment the workgroups together read one
+  // contiguous window of W (gridDim.x tiles of 16 rows), which spreads evenly over the memory channels
+  const int tiles = d.N / 16;
+  const int G = gridDim.x, t_first = blockIdx.x;
+  const int t_count = t_first < tiles ? (tiles - t_first + G - 1) / G : 0;
+  if (t_count == 0) return;                    // uniform per workgroup
+
+  // ---- resident X: rows 16 mh + r, K-steps q SPW .. of it, requested before the W stream ----------------
+  v8i xf[SPW];
+  int xs[SPW / 4];
+  {
+    const int m = 16 * mh + r;
+    const bool mok = m < d.M;
+    const uint8_t* const xrow = d.X + (int64_t)(mok ? m : 0) * d.ldx + (int64_t)q * SPW * 128 + gq * 16;
+    const uint8_t* const xsrow = d.Xs + (int64_t)(mok ? m : 0) * d.ldxs + q * SPW * 4;
+    v4i xlo[SPW], xhi[SPW], xsraw[SPW / 4];
+#pragma unroll
+    for (int s = 0; s < SPW; ++s) {
+      xlo[s] = *(const v4i*)(xrow + s * 128);
+      xhi[s] = *(const v4i*)(xrow + s * 128 + 64);
+    }
+#pragma unroll
+    for (int u = 0; u < SPW / 4; ++u) xsraw[u] = *(const v4i*)(xsrow + u * 16);
+    __builtin_amdgcn_sched_barrier(0);
+    issue(t_first, 0);
+    if (t_count > 1) issue(t_first + G, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    // operand form; rows beyond M are zeros with scale 1.0
+#pragma unroll
+    for (int s = 0; s < SPW; ++s) {
+      const v4i lo = xlo[s], hi = xhi[s];
+      xf[s] = mok ? (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w} : (v8i){0, 0, 0, 0, 0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int u = 0; u < SPW / 4; ++u) {
+      uint32_t pk = 0;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const uint32_t byte = mok ? (((uint32_t)xsraw[u][t] >> (8 * gq)) & 0xFFu) : 127u;
+        pk |= byte << (8 * t);
+      }
+      xs[u] = (int)pk;
+    }
+  }
+
+  for (int tb = 0; tb < t_count; tb += kBatch) {   // local tile index; uniform per workgroup
+    const int nt = t_count - tb < kBatch ? t_count - tb : kBatch;
+    v4f acc[kBatch];
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+    if (tb != 0) {                                      // the first batch was started above
+      issue(t_first + tb * G, 0);
+      if (nt > 1) issue(t_first + (tb + 1) * G, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      if (i < nt) {                                     // uniform
+        // this wave's share of tile i has landed (its share of tile i + 1 may stay in flight) ...
+        if (i + 1 < nt) {
+          if (with_scales) __builtin_amdgcn_s_waitcnt(0x0F70 | (Cf::WIW + 1));
+          else __builtin_amdgcn_s_waitcnt(0x0F70 | Cf::WIW);
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_barrier" ::: "memory");         // ... and so has everybody else's
+        __builtin_amdgcn_sched_barrier(0);
+        lds_u8* const wt = smem + (i & 1) * Cf::SLOT + q * (16 * Cf::SLB);
+        lds_u8* const st = smem + (i & 1) * Cf::SLOT + Cf::W_BYTES + r * Cf::SROW + q * (SPW * 4);
+        v4i sc[SPW / 4];
+#pragma unroll
+        for (int h = 0; h < SPW / 4; ++h) sc[h] = *(lds_cv4i*)(st + 16 * h);
+#pragma unroll
+        for (int s = 0; s < SPW; ++s) {
+          const v4i w = *(lds_cv4i*)(wt + r * Cf::SLB + (((s * 4 + gq) ^ r) << 4));
+          const v8i wf = {w.x, w.y, w.z, w.w, 0, 0, 0, 0};
+          const int wscale = (int)((uint32_t)sc[s / 4][s % 4] >> (8 * gq));
+          if (s % 4 == 0)
+            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], acc[i], MX_E2M1, XF, 0, wscale, 0, xs[s / 4]);
+          else if (s % 4 == 1)
+            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], acc[i], MX_E2M1, XF, 0, wscale, 1, xs[s / 4]);
+          else if (s % 4 == 2)
+            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], acc[i], MX_E2M1, XF, 0, wscale, 2, xs[s / 4]);
+          else
+            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], acc[i], MX_E2M1, XF, 0, wscale, 3, xs[s / 4]);
+        }
+        // every wave has its fragments of the slot in registers: refill it two tiles ahead
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        if (i + 2 < nt) issue(t_first + (tb + i + 2) * G, i & 1);
+      }
+    }
+
+    // ---- reduce the 4 K-slices of each half of M: partial sums meet in LDS (the ring is idle now) --------
+    lds_v4f* const red = (lds_v4f*)smem;
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i)
+      if (i < nt) red[(wave * kBatch + i) * 64 + lane] = acc[i];
+    __syncthreads();
+    const bool vec_ok = (d.ldc % 4 == 0) && (((uintptr_t)d.C) % 16 == 0);
+    for (int it = tid; it < nt * 128; it += kWaves * 64) {
+      const int i = it >> 7, h = (it >> 6) & 1, l = it & 63;
+      v4f sum = red[((h * 4 + 0) * kBatch + i) * 64 + l];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) sum += red[((h * 4 + w) * kBatch + i) * 64 + l];
+      // lane (c, g) of tile i holds C[16 h + c][16 tile + 4 g + e], e = 0..3
+      const int row = 16 * h + (l & 15);
+      if (row < d.M) {
+        OutT* c = (OutT*)d.C + (int64_t)row * d.ldc + (t_first + (tb + i) * G) * 16 + 4 * (l >> 4);
+        if constexpr (sizeof(OutT) == 4) {
+          if (vec_ok) {
+            if (d.accumulate) sum += *(const v4f*)c;
+            *(v4f*)c = sum;
+          } else {
+            for (int e = 0; e < 4; ++e) c[e] = d.accumulate ? c[e] + sum[e] : sum[e];
+          }
+        } else {
+          if (vec_ok) {
+            if (d.accumulate) {
+              const uint2 old = *(const uint2*)c;
+              sum.x += bf16_to_f32((uint16_t)old.x); sum.y += bf16_to_f32((uint16_t)(old.x >> 16));
+              sum.z += bf16_to_f32((uint16_t)old.y); sum.w += bf16_to_f32((uint16_t)(old.y >> 16));
+            }
+            uint2 o;
+            o.x = (uint32_t)f32_to_bf16(sum.x) | ((uint32_t)f32_to_bf16(sum.y) << 16);
+            o.y = (uint32_t)f32_to_bf16(sum.z) | ((uint32_t)f32_to_bf16(sum.w) << 16);
+            *(uint2*)c = o;
+          } else {
+            for (int e = 0; e < 4; ++e)
+              c[e] = f32_to_bf16(d.accumulate ? bf16_to_f32(c[e]) + sum[e] : sum[e]);
+          }
+        }
+      }
+    }
+    if (tb + kBatch < t_count) __syncthreads();   // the next batch's DMA overwrites the reduction buffer
+  }
+}
+
+template <int XF, int SPW, typename OutT>
+int launch_decode2_k(const DecodeArgs& d, int grid, hipStream_t stream) {
+  using Cf = Decode2Cfg<SPW>;
+  auto kern = decode2_kernel<XF, SPW, OutT>;
+  static int attr_done = 0;   // benign race: the attribute call is idempotent
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);
+    if (e != hipSuccess)
+      return set_error(MX_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", Cf::LDS_BYTES, hipGetErrorString(e));
+    attr_done = 1;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kWaves * 64), Cf::LDS_BYTES, stream, d);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "decode2_kernel launch: %s", hipGetErrorString(e));
+  return MX_OK;
+}
+
+template <int XF>
+int launch_decode2_x(const DecodeArgs& d, int grid, hipStream_t stream) {
+  if (d.K == 8192)
+    return d.c_dtype == MX_F32 ? launch_decode2_k<XF, 16, float>(d, grid, stream)
+                               : launch_decode2_k<XF, 16, uint16_t>(d, grid, stream);
+  return d.c_dtype == MX_F32 ? launch_decode2_k<XF, 8, float>(d, grid, stream)
+                             : launch_decode2_k<XF, 8, uint16_t>(d, grid, stream);
+}
+
 template <int XF, int SPW, int MT, typename OutT>
 int launch_decode_k(const DecodeArgs& d, int grid, hipStream_t stream) {
   using Cf = DecodeCfg<SPW, MT>;
@@ -318,6 +548,10 @@ int launch_gemm_decode(const DecodeArgs& d, hipStream_t stream) {
   const int tiles = d.N / 16;
   const int grid = tiles < 256 ? tiles : 256;
   if (grid == 0) return MX_OK;
+  // the two-halves variant where it applies (both halves of M in use, whole K-slices of 1024 or 2048)
+  static const int two_env = [] { const char* e = getenv("MXGEMM_DECODE2"); return e ? atoi(e) : 1; }();
+  if (two_env && d.M > 16 && (d.K == 8192 || d.K == 4096))
+    return d.x_fmt == MX_E4M3 ? launch_decode2_x<MX_E4M3>(d, grid, stream) : launch_decode2_x<MX_E5M2>(d, grid, stream);
   if (d.x_fmt == MX_E4M3) return launch_decode_x<MX_E4M3>(d, grid, stream);
   return launch_decode_x<MX_E5M2>(d, grid, stream);
 }

@@ -9,7 +9,8 @@ from oracle import mx_oracle as O
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("M,N,K", [(32, 256, 1024), (7, 1792, 2048), (16, 48, 512), (32, 4096, 8192), (1, 16, 4096)])
+@pytest.mark.parametrize("M,N,K", [(32, 256, 1024), (7, 1792, 2048), (16, 48, 512), (32, 4096, 8192), (1, 16, 4096),
+                                   (17, 4176, 4096), (29, 12320, 8192), (32, 16, 8192), (24, 36864, 4096)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=str)
 def test_decode_kernel(ct, dev, M, N, K, out_dtype):
     x = randn_operand(M, K, O.E4M3, 81, dev)
@@ -85,7 +86,23 @@ def test_grouped_gemm_sample_shape(ct, dev, kernel, tile, out_dtype):
     assert err <= (1e-3 if out_dtype == torch.float32 else 8e-3)
 
 
-@pytest.mark.parametrize("kernel", ["generic", "mfma128", "mfma256"])
+@pytest.mark.parametrize("K,x_fmt", [(4096, O.E4M3), (8192, O.E4M3)])
+def test_decode_two_halves_accumulate(ct, dev, K, x_fmt):
+    """16 < M <= 32 at K = 4096 / 8192 runs the variant whose waves split M as well as K: E5M2 activations,
+    C += into fp32 and bf16 (test_decode_kernel covers the ragged and the more-than-one-batch tile splits)."""
+    M, N = 27, 16 * 300
+    x = randn_operand(M, K, x_fmt, 86, dev)
+    w = randn_operand(N, K, O.E2M1, 87, dev, std=0.02)
+    ref = oracle_matmul(x, w)
+    for out_dtype, tol in ((torch.float32, 1e-3), (torch.bfloat16, 8e-3)):
+        z = torch.randn((M, N), generator=torch.Generator().manual_seed(88)).to(out_dtype)
+        acc = z.to(dev)
+        ct.block_scaled_matmul(x.storage, x.scale_t, w.storage.T, w.scale_t.T, b_format="e2m1", C=acc,
+                               accumulate=True, kernel="decode")
+        assert O.rel_fro(acc.float().cpu(), ref + z.float()) <= tol
+
+
+@pytest.mark.parametrize("kernel", ["generic", "mfma128", "mfma256", "pingpong"])
 def test_grouped_gemm_routed_weight_replicas1_and_padded_ids(ct, dev, kernel):
     """Second GEMM of the sample: replicas = 1, rows multiplied by the routed weight
     (test/kernels/fused_moe.py:75-77); index arrays left at their worst-case length."""
@@ -102,6 +119,10 @@ def test_grouped_gemm_routed_weight_replicas1_and_padded_ids(ct, dev, kernel):
         ct.invoke_fused_moe_scaled(a.storage, a.scale_t, W, ct.pack_scales(Ws), C2, wts.to(dev), sid, eid, True, 1,
                                    256, kernel=kernel)
         assert torch.equal(C, C2)
+        # bf16 output (the full-vector store path of the scatter epilogue where the tile's columns are inside N)
+        C3 = torch.zeros((T * topk, N), device=dev, dtype=torch.bfloat16)
+        ct.invoke_fused_moe_scaled(a.storage, a.scale_t, W, Ws, C3, wts.to(dev), sid, eid, True, 1, 256, kernel=kernel)
+        assert O.rel_fro(C3.float().cpu(), ref * wts.reshape(-1, 1)) < 8e-3
 
 
 @pytest.mark.parametrize("kernel,tile_m", [("auto", 128), ("auto", 256), ("generic", 16)])
