@@ -275,24 +275,31 @@ struct Decode2Cfg {
   static constexpr int W_BYTES = 4 * 16 * SLB;
   static constexpr int SLOT = W_BYTES + 16 * SROW;
   static constexpr int RING = 2 * SLOT;
-  static constexpr int RED = kWaves * kBatch * 64 * 16;
-  static constexpr int LDS_BYTES = RING > RED ? RING : RED;
+  static constexpr int RED = kWaves * 64 * 16;       // partial sums of one tile: [wave][lane] float4
+  static constexpr int LDS_BYTES = RING + 2 * RED;   // two reduction buffers behind the ring
 };
 
+// The weight and scale DMA of one wave for one tile.  Instruction j of the wave covers rows
+// rbase + j * RPI ... of the tile; lane offsets: row_off = (lane / LPR) * ldw, chunk_off = the lane's 16-byte
+// chunk position already XORed with its row inside the instruction (plus the K-slice's byte offset); the
+// instruction's first row enters the swizzle as one more XOR (rbase + RPI * j and lane / LPR share no bits).
 template <int SPW>
 __device__ inline void issue_tile_dma2(const uint8_t* W, uint32_t wbytes, const uint8_t* S, uint32_t sbytes,
-                                       lds_u8* wdst, lds_u8* sdst, const uint32_t* woff, uint32_t soff,
-                                       int wsoff, int ssoff, bool with_scales) {
+                                       lds_u8* wdst, lds_u8* sdst, uint32_t row_off, uint32_t chunk_off, int rbase,
+                                       uint32_t soff, int wsoff, int ldw, int ssoff, bool with_scales) {
   using Cf = Decode2Cfg<SPW>;
   const __amdgpu_buffer_rsrc_t rsW = make_rsrc(W, wbytes), rsS = make_rsrc(S, sbytes);
 #pragma unroll
-  for (int j = 0; j < Cf::WIW; ++j)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsW, (lds_void*)(wdst + j * 1024), 16, woff[j], wsoff, 0, 0);
+  for (int j = 0; j < Cf::WIW; ++j) {
+    const int r0 = rbase + j * Cf::RPI;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsW, (lds_void*)(wdst + j * 1024), 16,
+                                             row_off + (chunk_off ^ (uint32_t)((r0 & 15) << 4)), wsoff + r0 * ldw, 0, 0);
+  }
   if (with_scales)   // uniform per wave
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsS, (lds_void*)sdst, 16, soff, ssoff, 0, 0);
 }
 
-template <int XF, int SPW, typename OutT>
+template <int XF, int SPW, typename OutT, int VAR = 0>
 __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d) {
   using Cf = Decode2Cfg<SPW>;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
@@ -305,19 +312,15 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
 
   // ---- per-lane DMA offsets inside a tile --------------------------------------------------------------
   const uint32_t wbytes = (uint32_t)((int64_t)d.N * d.ldw), sbytes = (uint32_t)((int64_t)d.N * d.ldws);
-  uint32_t woff[Cf::WIW];
-#pragma unroll
-  for (int j = 0; j < Cf::WIW; ++j) {
-    const int rr = (mh * Cf::WIW + j) * Cf::RPI + lane / Cf::LPR, p = lane % Cf::LPR;
-    const int c = p ^ (rr & 15);               // chunk of the row that lives at LDS position p
-    woff[j] = (uint32_t)(rr * d.ldw + q * Cf::SLB + c * 16);
-  }
+  const int rl = lane / Cf::LPR;                 // row of the lane inside one DMA instruction
+  const uint32_t row_off = (uint32_t)(rl * d.ldw);
+  const uint32_t chunk_off = (uint32_t)((((lane % Cf::LPR) ^ rl) << 4) + q * Cf::SLB);   // SLB: no bits below 512
   const uint32_t soff = (uint32_t)((wave * (64 / Cf::LS) + lane / Cf::LS) * d.ldws + (lane % Cf::LS) * 16);
   auto issue = [&](int tile, int slot) {
     lds_u8* const base = smem + slot * Cf::SLOT;
     issue_tile_dma2<SPW>(d.W, wbytes, d.Ws, sbytes, base + q * (16 * Cf::SLB) + mh * Cf::WIW * 1024,
-                         base + Cf::W_BYTES + wave * 1024, woff, soff, tile * 16 * (int)d.ldw,
-                         tile * 16 * (int)d.ldws, with_scales);
+                         base + Cf::W_BYTES + wave * 1024, row_off, chunk_off, mh * Cf::WIW * Cf::RPI, soff,
+                         tile * 16 * (int)d.ldw, (int)d.ldw, tile * 16 * (int)d.ldws, with_scales);
   };
 
   // tiles of this workgroup: blockIdx.x, + gridDim.x, ... -- at any moment the workgroups together read one
@@ -328,141 +331,168 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
   if (t_count == 0) return;                    // uniform per workgroup
 
   // ---- resident X: rows 16 mh + r, K-steps q SPW .. of it, requested before the W stream ----------------
+  // Buffer loads: rows at or beyond M are out of range and read as zeros (elements 0, scale byte 0 = 2^-127),
+  // so the operand registers are written by the loads themselves, with no masking pass over them.
   v8i xf[SPW];
   int xs[SPW / 4];
   {
+    const __amdgpu_buffer_rsrc_t rsX = make_rsrc(d.X, (uint32_t)((int64_t)d.M * d.ldx));
+    const __amdgpu_buffer_rsrc_t rsXs = make_rsrc(d.Xs, (uint32_t)((int64_t)d.M * d.ldxs));
     const int m = 16 * mh + r;
-    const bool mok = m < d.M;
-    const uint8_t* const xrow = d.X + (int64_t)(mok ? m : 0) * d.ldx + (int64_t)q * SPW * 128 + gq * 16;
-    const uint8_t* const xsrow = d.Xs + (int64_t)(mok ? m : 0) * d.ldxs + q * SPW * 4;
-    v4i xlo[SPW], xhi[SPW], xsraw[SPW / 4];
+    const uint32_t xoff = (uint32_t)(m * d.ldx + q * SPW * 128 + gq * 16);
+    const uint32_t xsoff = (uint32_t)(m * d.ldxs + q * SPW * 4);
+    v4i xsraw[SPW / 4];
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
-      xlo[s] = *(const v4i*)(xrow + s * 128);
-      xhi[s] = *(const v4i*)(xrow + s * 128 + 64);
+      v4i lo, hi;
+      if constexpr ((VAR & 4) != 0) { lo = (v4i){s, 1, 2, 3}; hi = lo; }
+      else {
+        lo = __builtin_amdgcn_raw_buffer_load_b128(rsX, xoff, s * 128, 0);
+        hi = __builtin_amdgcn_raw_buffer_load_b128(rsX, xoff, s * 128 + 64, 0);
+      }
+      xf[s] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     }
 #pragma unroll
-    for (int u = 0; u < SPW / 4; ++u) xsraw[u] = *(const v4i*)(xsrow + u * 16);
+    for (int u = 0; u < SPW / 4; ++u) {
+      if constexpr ((VAR & 4) != 0) { xsraw[u] = (v4i){u, 1, 2, 3}; continue; }
+      xsraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rsXs, xsoff, u * 16, 0);
+    }
     __builtin_amdgcn_sched_barrier(0);
     issue(t_first, 0);
     if (t_count > 1) issue(t_first + G, 1);
     __builtin_amdgcn_sched_barrier(0);
-    // operand form; rows beyond M are zeros with scale 1.0
-#pragma unroll
-    for (int s = 0; s < SPW; ++s) {
-      const v4i lo = xlo[s], hi = xhi[s];
-      xf[s] = mok ? (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w} : (v8i){0, 0, 0, 0, 0, 0, 0, 0};
-    }
 #pragma unroll
     for (int u = 0; u < SPW / 4; ++u) {
       uint32_t pk = 0;
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const uint32_t byte = mok ? (((uint32_t)xsraw[u][t] >> (8 * gq)) & 0xFFu) : 127u;
-        pk |= byte << (8 * t);
-      }
+      for (int t = 0; t < 4; ++t) pk |= (((uint32_t)xsraw[u][t] >> (8 * gq)) & 0xFFu) << (8 * t);
       xs[u] = (int)pk;
     }
   }
 
-  for (int tb = 0; tb < t_count; tb += kBatch) {   // local tile index; uniform per workgroup
-    const int nt = t_count - tb < kBatch ? t_count - tb : kBatch;
-    v4f acc[kBatch];
+  // ---- per tile: partial sums of the 4 K-slices meet in LDS and leave while the next tiles stream in -------
+  const bool vec_ok = (d.ldc % 4 == 0) && (((uintptr_t)d.C) % 16 == 0);
+  auto reduce_store = [&](int k) {   // local tile k; threads 0 .. 127: half of M = tid / 64, lane l = tid % 64
+    lds_v4f* const red = (lds_v4f*)(smem + Cf::RING + (k & 1) * Cf::RED);
+    const int h = tid >> 6, l = tid & 63;
+    v4f sum = red[(h * 4 + 0) * 64 + l];
 #pragma unroll
-    for (int i = 0; i < kBatch; ++i) acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
-    if (tb != 0) {                                      // the first batch was started above
-      issue(t_first + tb * G, 0);
-      if (nt > 1) issue(t_first + (tb + 1) * G, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i) {
-      if (i < nt) {                                     // uniform
-        // this wave's share of tile i has landed (its share of tile i + 1 may stay in flight) ...
-        if (i + 1 < nt) {
-          if (with_scales) __builtin_amdgcn_s_waitcnt(0x0F70 | (Cf::WIW + 1));
-          else __builtin_amdgcn_s_waitcnt(0x0F70 | Cf::WIW);
-        } else {
-          __builtin_amdgcn_s_waitcnt(0x0F70);
+    for (int w = 1; w < 4; ++w) sum += red[(h * 4 + w) * 64 + l];
+    // lane (c, g) holds C[16 h + c][16 tile + 4 g + e], e = 0..3
+    const int row = 16 * h + (l & 15);
+    if (row >= d.M) return;
+    OutT* c = (OutT*)d.C + (int64_t)row * d.ldc + (t_first + k * G) * 16 + 4 * (l >> 4);
+    if constexpr (sizeof(OutT) == 4) {
+      if (vec_ok) {
+        if (d.accumulate) sum += *(const v4f*)c;
+        *(v4f*)c = sum;
+      } else {
+        for (int e = 0; e < 4; ++e) c[e] = d.accumulate ? c[e] + sum[e] : sum[e];
+      }
+    } else {
+      if (vec_ok) {
+        if (d.accumulate) {
+          const uint2 old = *(const uint2*)c;
+          sum.x += bf16_to_f32((uint16_t)old.x); sum.y += bf16_to_f32((uint16_t)(old.x >> 16));
+          sum.z += bf16_to_f32((uint16_t)old.y); sum.w += bf16_to_f32((uint16_t)(old.y >> 16));
         }
-        __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_barrier" ::: "memory");         // ... and so has everybody else's
-        __builtin_amdgcn_sched_barrier(0);
-        lds_u8* const wt = smem + (i & 1) * Cf::SLOT + q * (16 * Cf::SLB);
-        lds_u8* const st = smem + (i & 1) * Cf::SLOT + Cf::W_BYTES + r * Cf::SROW + q * (SPW * 4);
-        v4i sc[SPW / 4];
-#pragma unroll
-        for (int h = 0; h < SPW / 4; ++h) sc[h] = *(lds_cv4i*)(st + 16 * h);
-#pragma unroll
-        for (int s = 0; s < SPW; ++s) {
-          const v4i w = *(lds_cv4i*)(wt + r * Cf::SLB + (((s * 4 + gq) ^ r) << 4));
-          const v8i wf = {w.x, w.y, w.z, w.w, 0, 0, 0, 0};
-          const int wscale = (int)((uint32_t)sc[s / 4][s % 4] >> (8 * gq));
-          if (s % 4 == 0)
-            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], acc[i], MX_E2M1, XF, 0, wscale, 0, xs[s / 4]);
-          else if (s % 4 == 1)
-            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], acc[i], MX_E2M1, XF, 0, wscale, 1, xs[s / 4]);
-          else if (s % 4 == 2)
-            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], acc[i], MX_E2M1, XF, 0, wscale, 2, xs[s / 4]);
-          else
-            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], acc[i], MX_E2M1, XF, 0, wscale, 3, xs[s / 4]);
-        }
-        // every wave has its fragments of the slot in registers: refill it two tiles ahead
-        __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-        if (i + 2 < nt) issue(t_first + (tb + i + 2) * G, i & 1);
+        uint2 o;
+        o.x = (uint32_t)f32_to_bf16(sum.x) | ((uint32_t)f32_to_bf16(sum.y) << 16);
+        o.y = (uint32_t)f32_to_bf16(sum.z) | ((uint32_t)f32_to_bf16(sum.w) << 16);
+        *(uint2*)c = o;
+      } else {
+        for (int e = 0; e < 4; ++e)
+          c[e] = f32_to_bf16(d.accumulate ? bf16_to_f32(c[e]) + sum[e] : sum[e]);
       }
     }
+  };
 
-    // ---- reduce the 4 K-slices of each half of M: partial sums meet in LDS (the ring is idle now) --------
-    lds_v4f* const red = (lds_v4f*)smem;
+  for (int i = 0; i < t_count; ++i) {   // uniform per workgroup
+    // this wave's share of tile i has landed (its share of tile i + 1 may stay in flight) ...
+    if (i + 1 < t_count) {
+      if (with_scales) __builtin_amdgcn_s_waitcnt(0x0F70 | (Cf::WIW + 1));
+      else __builtin_amdgcn_s_waitcnt(0x0F70 | Cf::WIW);
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // ... and so has everybody else's; the partial sums of tile i - 1 are all in LDS as well
+    if constexpr (!(VAR & 8)) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    // all of the tile's fragments and scales into registers, so that the slot can be refilled before the
+    // multiplications start.  The scales first, packed to the lane's own byte of each K-step (one register
+    // per four K-steps): with the 16 raw scale registers alive next to the fragments the kernel would spill,
+    // and a spill reload queues behind the DMA just issued.
+    lds_u8* const wt = smem + (i & 1) * Cf::SLOT + q * (16 * Cf::SLB) + r * Cf::SLB;
+    lds_u8* const st = smem + (i & 1) * Cf::SLOT + Cf::W_BYTES + r * Cf::SROW + q * (SPW * 4);
+    int ws[SPW / 4];
+    v4i w[SPW];
+    if constexpr (!(VAR & 1)) {
 #pragma unroll
-    for (int i = 0; i < kBatch; ++i)
-      if (i < nt) red[(wave * kBatch + i) * 64 + lane] = acc[i];
-    __syncthreads();
-    const bool vec_ok = (d.ldc % 4 == 0) && (((uintptr_t)d.C) % 16 == 0);
-    for (int it = tid; it < nt * 128; it += kWaves * 64) {
-      const int i = it >> 7, h = (it >> 6) & 1, l = it & 63;
-      v4f sum = red[((h * 4 + 0) * kBatch + i) * 64 + l];
+      for (int h = 0; h < SPW / 4; ++h) {
+        const v4i sc = *(lds_cv4i*)(st + 16 * h);
+        uint32_t pk = 0;
 #pragma unroll
-      for (int w = 1; w < 4; ++w) sum += red[((h * 4 + w) * kBatch + i) * 64 + l];
-      // lane (c, g) of tile i holds C[16 h + c][16 tile + 4 g + e], e = 0..3
-      const int row = 16 * h + (l & 15);
-      if (row < d.M) {
-        OutT* c = (OutT*)d.C + (int64_t)row * d.ldc + (t_first + (tb + i) * G) * 16 + 4 * (l >> 4);
-        if constexpr (sizeof(OutT) == 4) {
-          if (vec_ok) {
-            if (d.accumulate) sum += *(const v4f*)c;
-            *(v4f*)c = sum;
-          } else {
-            for (int e = 0; e < 4; ++e) c[e] = d.accumulate ? c[e] + sum[e] : sum[e];
-          }
-        } else {
-          if (vec_ok) {
-            if (d.accumulate) {
-              const uint2 old = *(const uint2*)c;
-              sum.x += bf16_to_f32((uint16_t)old.x); sum.y += bf16_to_f32((uint16_t)(old.x >> 16));
-              sum.z += bf16_to_f32((uint16_t)old.y); sum.w += bf16_to_f32((uint16_t)(old.y >> 16));
-            }
-            uint2 o;
-            o.x = (uint32_t)f32_to_bf16(sum.x) | ((uint32_t)f32_to_bf16(sum.y) << 16);
-            o.y = (uint32_t)f32_to_bf16(sum.z) | ((uint32_t)f32_to_bf16(sum.w) << 16);
-            *(uint2*)c = o;
-          } else {
-            for (int e = 0; e < 4; ++e)
-              c[e] = f32_to_bf16(d.accumulate ? bf16_to_f32(c[e]) + sum[e] : sum[e]);
-          }
-        }
+        for (int t = 0; t < 4; ++t) pk |= (((uint32_t)sc[t] >> (8 * gq)) & 0xFFu) << (8 * t);
+        ws[h] = (int)pk;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // chunk (4 s + g) ^ r = 16 (s / 4) + (4 ((s % 4) ^ (r / 4)) + (g ^ (r % 4))): four lane-dependent
+      // addresses, the rest is an immediate offset
+      lds_u8* wk[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) wk[k] = wt + ((4 * (k ^ (r >> 2)) + (gq ^ (r & 3))) << 4);
+#pragma unroll
+      for (int s = 0; s < SPW; ++s) w[s] = *(lds_cv4i*)(wk[s & 3] + (s >> 2) * 256);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!(VAR & 8)) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    if (i + 2 < t_count) issue(t_first + (i + 2) * G, i & 1);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!(VAR & 2))
+      if (i > 0 && wave < 2) reduce_store(i - 1);   // uniform per wave
+    v4f acc[2] = {(v4f){0.f, 0.f, 0.f, 0.f}, (v4f){0.f, 0.f, 0.f, 0.f}};   // even / odd K-steps: two MFMA chains
+    if constexpr (!(VAR & 1)) {
+#pragma unroll
+      for (int s = 0; s < SPW; ++s) {
+        const v8i wf = {w[s].x, w[s].y, w[s].z, w[s].w, 0, 0, 0, 0};
+        v4f& a = acc[s & 1];
+        if (s % 4 == 0)
+          a = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], a, MX_E2M1, XF, 0, ws[s / 4], 0, xs[s / 4]);
+        else if (s % 4 == 1)
+          a = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], a, MX_E2M1, XF, 1, ws[s / 4], 1, xs[s / 4]);
+        else if (s % 4 == 2)
+          a = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], a, MX_E2M1, XF, 2, ws[s / 4], 2, xs[s / 4]);
+        else
+          a = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[s], a, MX_E2M1, XF, 3, ws[s / 4], 3, xs[s / 4]);
       }
     }
-    if (tb + kBatch < t_count) __syncthreads();   // the next batch's DMA overwrites the reduction buffer
+    ((lds_v4f*)(smem + Cf::RING + (i & 1) * Cf::RED))[wave * 64 + lane] = acc[0] + acc[1];
   }
+  __syncthreads();
+  if constexpr (!(VAR & 2))
+    if (wave < 2) reduce_store(t_count - 1);
 }
 
 template <int XF, int SPW, typename OutT>
 int launch_decode2_k(const DecodeArgs& d, int grid, hipStream_t stream) {
   using Cf = Decode2Cfg<SPW>;
   auto kern = decode2_kernel<XF, SPW, OutT>;
+#ifdef MXGEMM_TIMING_AIDS
+  // Only in builds made with -DMXGEMM_TIMING_AIDS: MXGEMM_DEC selects a variant with parts of the work removed
+  // (results invalid): 1 no MFMA / LDS reads, 2 no reduction, 4 no X loads, 8 no barriers
+  static const int var = [] { const char* e = getenv("MXGEMM_DEC"); return e ? atoi(e) : 0; }();
+  if constexpr (SPW == 16 && sizeof(OutT) == 2) {
+    if (var == 1) kern = decode2_kernel<XF, SPW, OutT, 1>;
+    if (var == 2) kern = decode2_kernel<XF, SPW, OutT, 2>;
+    if (var == 3) kern = decode2_kernel<XF, SPW, OutT, 3>;
+    if (var == 4) kern = decode2_kernel<XF, SPW, OutT, 4>;
+    if (var == 6) kern = decode2_kernel<XF, SPW, OutT, 6>;
+    if (var == 7) kern = decode2_kernel<XF, SPW, OutT, 7>;
+    if (var != 0) hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);
+  }
+#endif
   static int attr_done = 0;   // benign race: the attribute call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);
