@@ -37,8 +37,8 @@ PEAK_TFLOPS = {"mxfp8": 5033.0, "mxfp4": 10066.0}   # MI355X dense MFMA peaks (v
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the headline GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # `bench.py --only c2 --calib-copy`, each scaled by what the same counter reads for the 256 MiB copy kernel
-# (summary under profiles/): 412266 KiB x 2.0 + 156000 KiB x 1.0
-C2_HBM_TRAFFIC_BYTES = 980532 * 1024
+# (summary under profiles/): 406187 KiB x 2.0 + 141436 KiB x 1.0
+C2_HBM_TRAFFIC_BYTES = 953810 * 1024
 METRIC = "MX GEMM TFLOP/s (+% MFMA peak) 8192^3 MXFP8/MXFP4; GB/s at M=32 decode"
 
 
@@ -301,6 +301,7 @@ def cpu_baseline_c2(O, sets, budget_s=12.0):
 
 
 def main():
+    global SETTLE_S
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
@@ -308,12 +309,15 @@ def main():
     ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c5 (default: all)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the correctness check before timing")
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_S * 1e3,
+                    help="untimed settle period before every timed region (0 for counter-collection runs)")
     ap.add_argument("--no-vendor", action="store_true",
                     help="skip the context leg that times torch._scaled_mm on the headline operands")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (a known-size reference for "
                          "scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     a = ap.parse_args()
+    SETTLE_S = a.settle_ms * 1e-3
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py: this build measures ONE GPU (the path has no cross-GPU exchange; a larger "
                          "job would shard the weights along N and run this same kernel per GPU); run with --gpus 1")
