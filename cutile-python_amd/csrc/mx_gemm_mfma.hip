@@ -299,10 +299,13 @@ int launch_one(const GemmArgs& g, hipStream_t stream) {
 template <int BM, int BN, int WGM, int WGN>
 int launch_fmt(const GemmArgs& g, hipStream_t stream) {
   const bool grouped = g.sorted_token_ids != nullptr;
-  // tuning aid: MXGEMM_PIPE=0 selects the variant that issues all DMA loads of a stage in one burst
+  GemmArgs gs = g;
+#ifdef MXGEMM_TIMING_AIDS
+  // Only in builds made with -DMXGEMM_TIMING_AIDS (never the shipped library): MXGEMM_PIPE selects a variant
+  // with parts of the work removed (results invalid, except 0: all DMA loads of a stage in one burst);
+  // MXGEMM_STAGGER=1 starts every tile at a different K-quad
   static const int pipe_env = [] { const char* e = getenv("MXGEMM_PIPE"); return e ? atoi(e) : 1; }();
   static const int stagger_env = [] { const char* e = getenv("MXGEMM_STAGGER"); return e ? atoi(e) : 0; }();
-  GemmArgs gs = g;
   gs.stagger = stagger_env;
   if (pipe_env != 1 && g.a_fmt == MX_E4M3 && g.b_fmt == MX_E4M3 && g.c_dtype == MX_BF16 && !grouped) {
     using C = Cfg<MX_E4M3, MX_E4M3, BM, BN, WGM, WGN>;
@@ -316,6 +319,7 @@ int launch_fmt(const GemmArgs& g, hipStream_t stream) {
       case 7: return launch_one<C, uint16_t, false, 7>(gs, stream);   // only the A loads
     }
   }
+#endif
 #define MX_CASE(AFMT, BFMT)                                                                        \
   if (g.a_fmt == AFMT && g.b_fmt == BFMT) {                                                        \
     using C = Cfg<AFMT, BFMT, BM, BN, WGM, WGN>;                                                   \
