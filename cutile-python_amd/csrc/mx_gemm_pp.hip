@@ -214,6 +214,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   const bool accumulate = g.accumulate != 0;
   int eid[2] = {-1, -1};
   auto write_tile = [&](int m0, int n0) {
+    if constexpr ((VAR & 16) != 0) walk.origin(walk.first, m0, n0);   // timing aid: every tile to the same place
     if constexpr (!GROUPED) {
       // interior tile, plain store: one address per lane, everything else immediate offsets
       if (m0 + 256 <= g.M && n0 + 256 <= g.N && vec_ok && !accumulate) {
@@ -317,8 +318,12 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     if constexpr (t0 == 0) {
       if (s == 0 && lid != walk.first) {
         // the previous tile's output leaves while the other team is in its MFMA phase
+        // (the tile index passes through an opaque move: otherwise the compiler computes the eight row
+        // pointers of the stores when the tile begins and keeps them in registers through all its stages)
+        int plid = lid - walk.step;
+        asm volatile("" : "+s"(plid));
         int pm0, pn0;
-        walk.origin(lid - walk.step, pm0, pn0);
+        walk.origin(plid, pm0, pn0);
         write_tile(pm0, pn0);
         if constexpr (GROUPED) {
           walk.origin(lid, pm0, pn0);
@@ -514,7 +519,8 @@ int launch_gemm_pingpong(const GemmArgs& g, hipStream_t stream) {
 #ifdef MXGEMM_TIMING_AIDS
   // Only in builds made with -DMXGEMM_TIMING_AIDS (never the shipped library): MXGEMM_PP_VAR, read once,
   // selects a variant with parts of the work removed (results invalid): 1 no DMA in the loop, 2 no output
-  // stores, 4 no late LDS reads, 8 DMA of cache-resident data
+  // stores, 4 no late LDS reads, 8 DMA of cache-resident data, 16 every tile of a workgroup stored to the
+  // place of its first one (cache-resident output)
   static const int var_env = [] { const char* e = getenv("MXGEMM_PP_VAR"); return e ? (int)strtol(e, nullptr, 0) : 0; }();
   if (var_env && g.a_fmt == MX_E4M3 && g.b_fmt == MX_E4M3 && g.c_dtype == MX_BF16) {
     using C = Cfg<MX_E4M3, MX_E4M3, 256, 256, 2, 4>;
@@ -537,6 +543,7 @@ int launch_gemm_pingpong(const GemmArgs& g, hipStream_t stream) {
         case 7: return launch_pp<C, uint16_t, false, 7>(g, stream);
         case 8: return launch_pp<C, uint16_t, false, 8>(g, stream);
         case 10: return launch_pp<C, uint16_t, false, 10>(g, stream);
+        case 16: return launch_pp<C, uint16_t, false, 16>(g, stream);
       }
     }
   }
