@@ -49,7 +49,7 @@ struct PP {
   static constexpr int A_RPI = 64 / C::A_CPR, B_RPI = 64 / C::B_CPR;   // rows per DMA instruction
   static constexpr int AL = 128 / A_RPI / 4;                // A loads per wave and stage
   static constexpr int BL = 64 / B_RPI;                     // B loads per team-1 wave and stage
-  static constexpr int SCALE_LOADS = 3;                     // two A groups, one B group
+  static constexpr int SCALE_LOADS = 6;                     // two A groups (16 bytes each), four B tiles (4 bytes each)
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
@@ -64,14 +64,15 @@ template <typename OutT>
 __device__ __attribute__((noinline)) void write_tile_checked(AccTile t, OutT* Cp, int64_t ldc, int M, int N,
                                                              int mw, int nw, bool accumulate,
                                                              bool vec_ok) {
-  // mw / nw: row of the lane in tile (0, j) / first column of the lane in tile (i, 0)
+  // mw / nw: row of the lane in tile (0, j) / first column of the lane in tile (i, 0); tile (i, j) starts
+  // bperm_tile_off(j) columns further
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int m = mw + 16 * i;
     if (m >= M) continue;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int n = nw + 16 * j;
+      const int n = nw + bperm_tile_off(j);
       if (n >= N) continue;
       store4<OutT>(Cp + (int64_t)m * ldc + n, t.v[i][j], accumulate, N - n, vec_ok);
     }
@@ -115,18 +116,27 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
 
   // ---- load context: where the DMA and scale loads of the tile being FETCHED point --------------------
   // A: instruction q of the wave covers tile rows wm0 + (4 q + wn) * A_RPI ...; B (team 1 only):
-  // rows wn0 + q * B_RPI ....  The swizzled byte column of instruction q is col0 ^ (4 q % CPR) * 16.
+  // rows wn0 + q * B_RPI ....  A: the swizzled byte column of instruction q is col0 ^ (4 q % CPR) * 16.
   uint32_t a_voff[AL], b_voff[TEAM ? BL : 1];
   const int a_row0 = wm0 + wn * P::A_RPI + lane / C::A_CPR;
   const int a_col0 = ((lane % C::A_CPR) ^ swz<C::A_CPR>(a_row0)) * 16;
   const int b_row0 = wn0 + lane / C::B_CPR;
-  const int b_col0 = ((lane % C::B_CPR) ^ swz<C::B_CPR>(b_row0)) * 16;
+  // swizzled byte column of DMA instruction q (rows b_row0 + q * B_RPI ...)
+  auto b_col = [&](int q) { return ((lane % C::B_CPR) ^ swz_bperm<C::B_CPR>(lane / C::B_CPR + q * P::B_RPI)) * 16; };
   __amdgpu_buffer_rsrc_t rsB;
   // scale groups (16-byte index of K-quad 0, lane 0) of this wave's rows / columns: for the tile being
   // computed and for the tile being fetched
   int as_cur[2], bs_cur, as_nxt[2], bs_nxt;
+  v4i sb;   // scale dwords of the wave's four B tiles for the current K-quad
   const v4i* const As4 = (const v4i*)g.As + lane;
-  const v4i* const Bs4 = (const v4i*)g.Bs + lane;
+  // B scales: tile j of this lane is B row bperm_row(j, r) = 16-row group 2 (j / 2) + r / 8 of the wave's 64 rows,
+  // row 8 (r / 4 % 2) + 4 (j % 2) + r % 4 inside it; in the packed layout ([64-row group][K-quad][lane][group % 4]
+  // dwords, lane = row % 16 + 16 * K-block) that is one dword per tile, 16 (j % 2) + 2 (j / 2) dwords apart
+  const int* const Bs1 = (const int*)g.Bs + 4 * (8 * ((r >> 2) & 1) + (r & 3) + 16 * gq) + (r >> 3);
+  auto load_b_scales = [&](int idx16) {   // idx16: 16-byte index of (64-row group, K-quad), lane 0
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sb[j] = Bs1[(int64_t)idx16 * 4 + 16 * (j & 1) + 2 * (j >> 1)];
+  };
   bool fetch_valid = true;   // false once the walk has no further tile: loads become zero-fill no-ops
   auto set_fetch_tile = [&](int lid) {
     fetch_valid = lid < walk.end;
@@ -150,7 +160,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     if constexpr (TEAM == 1) {
 #pragma unroll
       for (int q = 0; q < BL; ++q) {
-        const int col = b_col0 ^ (((4 * q) % C::B_CPR) << 4);
+        const int col = b_col(q);
         const int64_t grow = n0 + b_row0 + q * P::B_RPI;
         b_voff[q] = (fetch_valid && grow < g.N) ? (uint32_t)(grow * g.ldb + col) : kOobOffset;
       }
@@ -191,14 +201,14 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       const int klim = sl < nstages ? Kb_b - kb : 0;
 #pragma unroll
       for (int q = 0; q < BL; ++q) {
-        const int col = b_col0 ^ (((4 * q) % C::B_CPR) << 4);
+        const int col = b_col(q);
         const uint32_t v = col >= klim ? kOobOffset : b_voff[q];
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(base + q * 1024), 16, v, kb, 0, 0);
       }
     }
   };
 
-  v4i sa[2], sb;
+  v4i sa[2];
   v4f acc[8][4];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
@@ -207,24 +217,27 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   const int swa = swz<C::A_CPR>(r), swb = swz<C::B_CPR>(r);
   constexpr int SPQ = 4 / C::KSUB;   // stages per K-quad
 
-  // ---- output of a finished tile: lane (c, g) of tile (i, j) holds rows 16 i + c, columns
-  // 16 j + 4 g .. + 3; the accumulators are cleared for the next tile ------------------------------------
+  // ---- output of a finished tile: lane (c, g) of tile (i, j) holds row 16 i + c, columns
+  // 32 (j / 2) + 8 g + 4 (j % 2) .. + 3 (see bperm_tile_off); the accumulators are cleared for the next tile ------------------------------------
   OutT* const Cp = (OutT*)g.C;
   const bool vec_ok = (g.ldc % 4 == 0) && (((uintptr_t)g.C) % 16 == 0);
+  // the lane's 8 consecutive outputs of a tile pair as 16-byte stores: every row start 16-byte aligned
+  const bool vec8_ok = ((g.ldc * (int64_t)sizeof(OutT)) % 16 == 0) && (((uintptr_t)g.C) % 16 == 0);
   const bool accumulate = g.accumulate != 0;
   int eid[2] = {-1, -1};
   auto write_tile = [&](int m0, int n0) {
     if constexpr ((VAR & 16) != 0) walk.origin(walk.first, m0, n0);   // timing aid: every tile to the same place
     if constexpr (!GROUPED) {
       // interior tile, plain store: one address per lane, everything else immediate offsets
-      if (m0 + 256 <= g.M && n0 + 256 <= g.N && vec_ok && !accumulate) {
-        OutT* p = Cp + (int64_t)(m0 + wm0 + r) * g.ldc + (n0 + wn0 + 4 * gq);
+      if (m0 + 256 <= g.M && n0 + 256 <= g.N && vec8_ok && !accumulate) {
+        OutT* p = Cp + (int64_t)(m0 + wm0 + r) * g.ldc + (n0 + wn0 + 8 * gq);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            if (!(VAR & 2) || g.ldc == -12345) store4_full<OutT>(p + 16 * j, acc[i][j]);
-            acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+          for (int jp = 0; jp < 2; ++jp) {
+            if (!(VAR & 2) || g.ldc == -12345) store8_full<OutT>(p + 32 * jp, acc[i][2 * jp], acc[i][2 * jp + 1]);
+            acc[i][2 * jp] = (v4f){0.f, 0.f, 0.f, 0.f};
+            acc[i][2 * jp + 1] = (v4f){0.f, 0.f, 0.f, 0.f};
           }
           p += 16 * g.ldc;
         }
@@ -239,12 +252,12 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
           acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
         }
       if (!(VAR & 2) || g.ldc == -12345)
-        write_tile_checked<OutT>(t, Cp, g.ldc, g.M, g.N, m0 + wm0 + r, n0 + wn0 + 4 * gq, accumulate, vec_ok);
+        write_tile_checked<OutT>(t, Cp, g.ldc, g.M, g.N, m0 + wm0 + r, n0 + wn0 + 8 * gq, accumulate, vec_ok);
       return;
     }
     // grouped: row 16 i + c of the team's half goes to row `id` of C, where id is the routed-slot index
     // that lane 16 (i % 4) + c of eid[i / 4] has held since the tile began (no load latency here)
-    const bool cols_in = n0 + 256 <= g.N && vec_ok && !accumulate;   // uniform
+    const bool cols_in = n0 + 256 <= g.N && vec8_ok && !accumulate;   // uniform
     float ewt[2] = {1.f, 1.f};
     if (g.topk_weights) {
 #pragma unroll
@@ -258,18 +271,18 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       const bool ok = id >= 0 && id < g.num_valid_ids;
       float w = 1.f;
       if (g.topk_weights) w = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, ewt[i >> 2])));
-      OutT* const p = Cp + (int64_t)id * g.ldc + (n0 + wn0 + 4 * gq);
+      OutT* const p = Cp + (int64_t)id * g.ldc + (n0 + wn0 + 8 * gq);
       if (cols_in) {
         if ((!(VAR & 2) || g.ldc == -12345) && ok) {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) store4_full<OutT>(p + 16 * j, acc[i][j] * w);
+          for (int jp = 0; jp < 2; ++jp) store8_full<OutT>(p + 32 * jp, acc[i][2 * jp] * w, acc[i][2 * jp + 1] * w);
         }
       } else {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const int n = n0 + wn0 + 16 * j + 4 * gq;
+          const int n = n0 + wn0 + 8 * gq + bperm_tile_off(j);
           if ((!(VAR & 2) || g.ldc == -12345) && ok && n < g.N)
-            store4<OutT>(p + 16 * j, acc[i][j] * w, accumulate, g.N - n, vec_ok);
+            store4<OutT>(p + bperm_tile_off(j), acc[i][j] * w, accumulate, g.N - n, vec_ok);
         }
       }
 #pragma unroll
@@ -301,7 +314,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   issue_b(1, 1);
 #pragma unroll
   for (int u = 0; u < 2; ++u) sa[u] = As4[as_nxt[u]];
-  sb = Bs4[bs_nxt];
+  load_b_scales(bs_nxt);
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_barrier" ::: "memory");
@@ -337,13 +350,13 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     const int sl = wrapped ? s + 2 - nstages : s + 2;   // local stage the loads fetch
     const int sl_eff = (wrapped && (!fetch_valid || nstages < 2)) ? nstages : sl;
     lds_u8* const atile = smem + abuf * C::A_STAGE + (wm0 + r) * C::A_RB;
-    lds_u8* const btile = smem + P::B_BASE + bbuf * C::B_STAGE + (wn0 + r) * C::B_RB;
+    lds_u8* const btile = smem + P::B_BASE + bbuf * C::B_STAGE + (wn0 + bperm_lane_off(r)) * C::B_RB;
     issue_a(sl_eff, abuf2);
     v8i bf[C::KSUB][4], af[C::KSUB][8];
 #pragma unroll
     for (int kk = 0; kk < C::KSUB; ++kk) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) bf[kk][j] = load_frag<C::B_RB, C::B_EB>(btile, 16 * j, kk, gq, swb);
+      for (int j = 0; j < 4; ++j) bf[kk][j] = load_frag<C::B_RB, C::B_EB>(btile, bperm_tile_off(j), kk, gq, swb);
 #pragma unroll
       for (int i = 0; i < EARLY; ++i) af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
     }
@@ -407,7 +420,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       const int Qk = more ? Q + 1 : 0;
 #pragma unroll
       for (int u = 0; u < 2; ++u) sa[u] = As4[(more ? as_cur[u] : as_nxt[u]) + Qk * 64];
-      sb = Bs4[(more ? bs_cur : bs_nxt) + Qk * 64];
+      load_b_scales((more ? bs_cur : bs_nxt) + Qk * 64);
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);

@@ -42,6 +42,23 @@ __device__ inline int swz(int row) {
   return (row / (16 / CPR)) % CPR;
 }
 
+// ---- column order of the ping-pong kernel's B fragments ------------------------------------------------
+// MFMA tile j (0..3) of a wave's 64 B rows takes, as its operand row c, B row
+//     bperm_row(j, c) = 32 (j / 2) + 8 (c / 4) + 4 (j % 2) + c % 4
+// instead of 16 j + c.  Lane (c, g) of the result then holds columns 32 (j / 2) + 8 g + 4 (j % 2) + e,
+// e = 0..3: the tiles j = 2p and 2p + 1 give it 8 consecutive outputs, which leave as one 16-byte (bf16) or
+// two adjacent 16-byte (fp32) stores -- half as many store instructions as with 4 consecutive outputs.
+__device__ inline int bperm_tile_off(int j) { return 32 * (j >> 1) + 4 * (j & 1); }   // part of the row that depends on j
+__device__ inline int bperm_lane_off(int c) { return 8 * (c >> 2) + (c & 3); }         // part that depends on the lane
+// LDS swizzle of the B rows for that read pattern: built from the row bits that tell the 16 lanes of a read
+// apart beyond the bank half (CPR = 8: bits 1, 3, 4; CPR = 4: bits 3, 4); for row bperm_row(j, c) it equals
+// swz<CPR>(c), whatever j is.
+template <int CPR>
+__device__ inline int swz_bperm(int row) {
+  if constexpr (CPR == 8) return ((row >> 1) & 1) | (((row >> 3) & 3) << 1);
+  else return (row >> 3) & (CPR - 1);
+}
+
 // Fragment of one 16-row tile for MFMA K-step kk of the stage, lane group gq, in the operand layout
 // described at the top of the file.  8-bit formats: two 16-byte chunks; 4-bit: one, in the low dwords.
 template <int RB, int EB>
@@ -121,6 +138,29 @@ __device__ inline void store4_full<uint16_t>(uint16_t* p, const v4f& v) {
   w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v.x, v.y}, b2));
   w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v.z, v.w}, b2));
   *(uint2*)p = w;
+}
+
+// eight consecutive outputs (two accumulator quads), no bounds, alignment or accumulate handling
+template <typename OutT>
+__device__ inline void store8_full(OutT* p, const v4f& v0, const v4f& v1);
+
+template <>
+__device__ inline void store8_full<float>(float* p, const v4f& v0, const v4f& v1) {
+  *(v4f*)p = v0;
+  *(v4f*)(p + 4) = v1;
+}
+
+template <>
+__device__ inline void store8_full<uint16_t>(uint16_t* p, const v4f& v0, const v4f& v1) {
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  u4 w;
+  w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v0.x, v0.y}, b2));
+  w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v0.z, v0.w}, b2));
+  w.z = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v1.x, v1.y}, b2));
+  w.w = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v1.z, v1.w}, b2));
+  *(u4*)p = w;
 }
 
 }  // namespace mx
