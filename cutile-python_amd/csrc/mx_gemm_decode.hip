@@ -2,9 +2,9 @@
 //
 // The problem is bound by streaming W (and its scales) from HBM exactly once, so the kernel is
 // organised around long contiguous reads and many bytes in flight, not around tile reuse:
-//   * a workgroup of 8 waves owns a contiguous run of 16-row tiles of W (64 KiB each at K = 8192);
+//   * a workgroup of 8 waves takes every gridDim.x-th 16-row tile of W (64 KiB each at K = 8192);
 //     wave w owns K-slice w (SPW MFMA K-steps of 128 elements) of every tile, so the 8 waves together
-//     read each tile, and tile after tile, as one contiguous stream;
+//     read a tile as one contiguous piece and the workgroups together one contiguous window of W;
 //   * W and its E8M0 scales go global -> LDS with buffer_load ... lds (no VGPR staging): two tiles per
 //     wave are in flight (144 KiB per CU) while the previous one is multiplied.  A wave only ever reads
 //     back what it loaded itself, so the streaming loop has no workgroup barrier, only s_waitcnt vmcnt;
@@ -92,12 +92,12 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
   issue_tile_dma<SPW>(d.W, wbytes, d.Ws, sbytes, my + (slot) * Cf::SLOT, woff, soff, (tile) * 16 * (int)d.ldw, \
                       (tile) * 16 * (int)d.ldws)
 
+  // tiles of this workgroup: blockIdx.x, + gridDim.x, ... -- at any moment the workgroups together read one
+  // contiguous window of W, which spreads evenly over the memory channels
   const int tiles = d.N / 16;
-  const int per = tiles / gridDim.x, rem = tiles % gridDim.x;
-  const int b = blockIdx.x;
-  const int t_begin = b * per + (b < rem ? b : rem);
-  const int t_end = t_begin + per + (b < rem ? 1 : 0);
-  if (t_begin >= t_end) return;                // uniform per workgroup
+  const int G = gridDim.x, t_first = blockIdx.x;
+  const int t_count = t_first < tiles ? (tiles - t_first + G - 1) / G : 0;
+  if (t_count == 0) return;                    // uniform per workgroup
 
   // ---- resident X fragments and scales ---------------------------------------------------------------
   // All loads are issued unconditionally from clamped addresses (no branches, so they overlap), and
@@ -130,8 +130,8 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
   // hold back the first MFMA for as long as that burst takes to drain.  Now the W stream starts: the first
   // two tiles of this workgroup.
   __builtin_amdgcn_sched_barrier(0);
-  MX_ISSUE_TILE(t_begin, 0);
-  if (t_begin + 1 < t_end) MX_ISSUE_TILE(t_begin + 1, 1);
+  MX_ISSUE_TILE(t_first, 0);
+  if (t_count > 1) MX_ISSUE_TILE(t_first + G, 1);
 
   __builtin_amdgcn_sched_barrier(0);
   // X into the MFMA operand layout; rows beyond M and K-steps beyond K become zeros (scale 1.0)
@@ -157,17 +157,17 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
     }
   }
 
-  for (int tb = t_begin; tb < t_end; tb += kBatch) {   // uniform per workgroup
-    const int nt = t_end - tb < kBatch ? t_end - tb : kBatch;
+  for (int tb = 0; tb < t_count; tb += kBatch) {   // local tile index; uniform per workgroup
+    const int nt = t_count - tb < kBatch ? t_count - tb : kBatch;
     v4f acc[kBatch][MT];
 #pragma unroll
     for (int i = 0; i < kBatch; ++i)
 #pragma unroll
       for (int m = 0; m < MT; ++m) acc[i][m] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-    if (tb != t_begin) {                                // the first batch was started above
-      MX_ISSUE_TILE(tb, 0);
-      if (nt > 1) MX_ISSUE_TILE(tb + 1, 1);
+    if (tb != 0) {                                      // the first batch was started above
+      MX_ISSUE_TILE(t_first + tb * G, 0);
+      if (nt > 1) MX_ISSUE_TILE(t_first + (tb + 1) * G, 1);
     }
 #pragma unroll
     for (int i = 0; i < kBatch; ++i) {
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
         }
         // the slot is free again once its fragments are in registers: refill it two tiles ahead
         __builtin_amdgcn_sched_barrier(0);
-        if (i + 2 < nt) MX_ISSUE_TILE(tb + i + 2, i & 1);
+        if (i + 2 < nt) MX_ISSUE_TILE(t_first + (tb + i + 2) * G, i & 1);
       }
     }
 
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
       // lane (c, g) of tile i holds C[16 m + c][16 tile + 4 g + e], e = 0..3
       const int row = 16 * m + (l & 15);
       if (row < d.M) {
-        OutT* c = (OutT*)d.C + (int64_t)row * d.ldc + (tb + i) * 16 + 4 * (l >> 4);
+        OutT* c = (OutT*)d.C + (int64_t)row * d.ldc + (t_first + (tb + i) * G) * 16 + 4 * (l >> 4);
         if constexpr (sizeof(OutT) == 4) {
           if (vec_ok) {
             if (d.accumulate) sum += *(const v4f*)c;
@@ -250,7 +250,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
         }
       }
     }
-    if (tb + kBatch < t_end) __syncthreads();   // the next batch's DMA overwrites the reduction buffer
+    if (tb + kBatch < t_count) __syncthreads();   // the next batch's DMA overwrites the reduction buffer
   }
 #undef MX_ISSUE_TILE
 }
