@@ -112,17 +112,18 @@ if hasattr(torch, "float4_e2m1fn_x2"):
 def desc(t: torch.Tensor, mx_dtype: int, packed_dim: int = -1) -> MxTensor:
     """Descriptor of a torch tensor.  ``packed_dim`` >= 0 marks an FP4 tensor whose storage holds two
     logical elements per byte along that dimension (the logical extent is doubled)."""
+    nd = t.dim()
+    shape = tuple(t.shape)
+    if packed_dim >= 0:
+        shape = tuple(n * 2 if i == packed_dim else n for i, n in enumerate(shape))
     d = MxTensor()
     d.ptr = t.data_ptr()
     d.dtype = mx_dtype
-    d.ndim = t.dim()
-    itemsize = t.element_size()
-    for i in range(t.dim()):
-        d.shape[i] = t.shape[i] * (2 if i == packed_dim else 1)
-        # strides are in units of the storage type; all sub-byte / byte formats are 1 byte wide
-        d.stride[i] = t.stride(i)
+    d.ndim = nd
+    d.shape[0:nd] = shape
+    # strides are in units of the storage type; all sub-byte / byte formats are 1 byte wide
+    d.stride[0:nd] = t.stride()
     d.packed_dim = packed_dim
-    assert itemsize in (1, 2, 4)
     return d
 
 

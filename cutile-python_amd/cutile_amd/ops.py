@@ -147,12 +147,12 @@ def _scale_desc(s, rows: int, K: int, block: int, is_b: bool):
 _WS_CACHE: dict = {}
 
 
-def _workspace(dev: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+def _workspace(dev: torch.device, nbytes: int, stream: Optional[int] = None) -> Optional[torch.Tensor]:
     """Scratch for the per-call scale re-layout: one buffer per (device, stream), grown on demand, so the
     hot path does not go through the allocator.  Kernels that use it are ordered on that stream."""
     if nbytes <= 0:
         return None
-    key = (dev.index, L.stream_ptr(dev))
+    key = (dev.index, L.stream_ptr(dev) if stream is None else stream)
     buf = _WS_CACHE.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
@@ -174,11 +174,15 @@ def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kerne
     o = _opts(accumulate, la, lb, kernel, block, split_k)
     lib = L.lib()
     need = lib.mx_gemm_workspace_bytes(M, N, K, ctypes.byref(o))
-    ws = _workspace(dev, need)
-    with torch.cuda.device(dev):
-        rc = lib.mx_gemm(ctypes.byref(dA), ctypes.byref(dAs), ctypes.byref(dB), ctypes.byref(dBs),
-                         ctypes.byref(dC), ctypes.byref(o), ws.data_ptr() if ws is not None else None,
-                         need, L.stream_ptr(dev))
+    stream = L.stream_ptr(dev)
+    ws = _workspace(dev, need, stream)
+    args = (ctypes.byref(dA), ctypes.byref(dAs), ctypes.byref(dB), ctypes.byref(dBs), ctypes.byref(dC),
+            ctypes.byref(o), ws.data_ptr() if ws is not None else None, need, stream)
+    if torch.cuda.current_device() == dev.index:
+        rc = lib.mx_gemm(*args)
+    else:
+        with torch.cuda.device(dev):
+            rc = lib.mx_gemm(*args)
     _check(rc)
     return C
 
