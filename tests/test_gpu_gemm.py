@@ -57,10 +57,12 @@ def test_gemm_aligned(ct, dev, kernel, fa, fb, out_dtype):
 
 @pytest.mark.parametrize("kernel", MFMA)
 @pytest.mark.parametrize("fa,fb", FORMATS, ids=lambda f: str(f))
-@pytest.mark.parametrize("M,N,K", [(300, 200, 160), (1, 1, 32), (129, 257, 96), (64, 700, 544)])
+@pytest.mark.parametrize("M,N,K", [(300, 200, 160), (1, 1, 32), (129, 257, 96), (64, 700, 544), (512, 772, 256),
+                                   (520, 1032, 512)])
 def test_gemm_ragged(ct, dev, kernel, fa, fb, M, N, K):
     """Edge tiles in M and N and a K that is a multiple of 32 but not of the K tile: zero padding of
-    test/kernels/scaled_matmul.py:66-104."""
+    test/kernels/scaled_matmul.py:66-104.  The last two shapes mix interior and edge tiles of the 256x256
+    kernels, once with an output pitch that allows their 16-byte bf16 stores (1032) and once without (772)."""
     a = randn_operand(M, K, fa, 21, dev)
     b = randn_operand(N, K, fb, 22, dev)
     for out_dtype in (torch.float32, torch.bfloat16):
