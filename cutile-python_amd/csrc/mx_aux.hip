@@ -269,7 +269,7 @@ __device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float
 
 // 8 lanes per 32-element block, 4 consecutive elements per lane; every thread handles kQuantUnroll units a
 // grid apart and requests all their inputs before it processes the first (memory-level parallelism).
-constexpr int kQuantUnroll = 1;
+constexpr int kQuantUnroll = 2;
 __global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
   const int64_t nthreads = (int64_t)gridDim.x * 256;
   const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
