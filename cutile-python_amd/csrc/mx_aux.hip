@@ -116,32 +116,49 @@ __device__ inline float silu_mul_f32(float a, float b) {
   return __fmul_rn(t, b);
 }
 
-// four consecutive elements starting at element index i (k0 + 3 < K checked by the caller for `vec`)
-__device__ inline void load4_as_f32(const void* p, int64_t i, int dtype, bool vec, int nvalid, float* v) {
+// EPL consecutive elements starting at element index i (all of them inside K checked by the caller for `vec`)
+template <int EPL>
+__device__ inline void load_as_f32_vec(const void* p, int64_t i, int dtype, bool vec, int nvalid, float* v) {
   if (vec && dtype == MX_F32) {
-    const v4f t = *(const v4f*)((const float*)p + i);
-    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+#pragma unroll
+    for (int h = 0; h < EPL / 4; ++h) {
+      const v4f t = *(const v4f*)((const float*)p + i + 4 * h);
+      v[4 * h + 0] = t.x; v[4 * h + 1] = t.y; v[4 * h + 2] = t.z; v[4 * h + 3] = t.w;
+    }
   } else if (vec && dtype == MX_BF16) {
-    const uint2 t = *(const uint2*)((const uint16_t*)p + i);
-    v[0] = bf16_to_f32((uint16_t)t.x); v[1] = bf16_to_f32((uint16_t)(t.x >> 16));
-    v[2] = bf16_to_f32((uint16_t)t.y); v[3] = bf16_to_f32((uint16_t)(t.y >> 16));
+    uint32_t t[EPL / 2];
+    if constexpr (EPL == 8) {
+      const v4i r = *(const v4i*)((const uint16_t*)p + i);
+      t[0] = (uint32_t)r.x; t[1] = (uint32_t)r.y; t[2] = (uint32_t)r.z; t[3] = (uint32_t)r.w;
+    } else {
+      const uint2 r = *(const uint2*)((const uint16_t*)p + i);
+      t[0] = r.x; t[1] = r.y;
+    }
+#pragma unroll
+    for (int h = 0; h < EPL / 2; ++h) {
+      v[2 * h] = bf16_to_f32((uint16_t)t[h]);
+      v[2 * h + 1] = bf16_to_f32((uint16_t)(t[h] >> 16));
+    }
   } else {
-    for (int e = 0; e < 4; ++e) v[e] = e < nvalid ? load_as_f32(p, i + e, dtype) : 0.f;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) v[e] = e < nvalid ? load_as_f32(p, i + e, dtype) : 0.f;
   }
 }
 
-// Where unit `gid` (8 consecutive units = one 32-element block, 4 consecutive elements per unit) lives.
+// Where unit `gid` lives: 32 / EPL consecutive units are one 32-element block, EPL consecutive elements per unit.
 struct QuantUnit {
   int64_t row, kb, k0;
   int sub;
   bool live;
 };
 
+template <int EPL>
 __device__ inline QuantUnit quant_unit(const QuantArgs& q, int64_t gid) {
+  constexpr int UPB = 32 / EPL;   // units (lanes) per block
   const int64_t KB = q.Kpad / 32;
   QuantUnit u;
-  const int64_t blk = gid >> 3;
-  u.sub = (int)(gid & 7);
+  const int64_t blk = gid / UPB;
+  u.sub = (int)(gid % UPB);
   u.live = blk < q.rows * KB;
   if (q.rows * KB < ((int64_t)1 << 31)) {   // uniform: 32-bit division is several times cheaper
     const uint32_t b32 = u.live ? (uint32_t)blk : 0u, kb32 = (uint32_t)KB;
@@ -151,39 +168,48 @@ __device__ inline QuantUnit quant_unit(const QuantArgs& q, int64_t gid) {
     u.row = u.live ? blk / KB : 0;
     u.kb = u.live ? blk % KB : 0;
   }
-  u.k0 = u.kb * 32 + u.sub * 4;
+  u.k0 = u.kb * 32 + u.sub * EPL;
   return u;
 }
 
-// the (at most) four input values of a unit; the fused producer applies silu(x) * up
+// the (at most) EPL input values of a unit; the fused producer applies silu(x) * up
+template <int EPL>
 __device__ inline void quant_load(const QuantArgs& q, const QuantUnit& u, float* v, float* w) {
-  for (int e = 0; e < 4; ++e) v[e] = w[e] = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) v[e] = w[e] = 0.f;
   if (!u.live) return;
   const int64_t base = u.row * q.x_ld + u.k0;
   const int esz = q.x_dtype == MX_F32 ? 4 : 2;
-  const int nvalid = q.K - u.k0 >= 4 ? 4 : (q.K > u.k0 ? (int)(q.K - u.k0) : 0);
-  const bool vec = nvalid == 4 && q.x_dtype != MX_F16 &&
-                   ((((uintptr_t)q.x) | ((uintptr_t)q.up) | (uintptr_t)(q.x_ld * esz)) & (4 * esz - 1)) == 0;
-  load4_as_f32(q.x, base, q.x_dtype, vec, nvalid, v);
-  if (q.up) load4_as_f32(q.up, base, q.x_dtype, vec, nvalid, w);
+  const int nvalid = q.K - u.k0 >= EPL ? EPL : (q.K > u.k0 ? (int)(q.K - u.k0) : 0);
+  // 16-byte loads: fp32 in EPL / 4 pieces, bf16 as one (EPL = 8) or an 8-byte one (EPL = 4)
+  const int align = (q.x_dtype == MX_F32 || EPL == 8) ? 16 : 8;
+  const bool vec = nvalid == EPL && q.x_dtype != MX_F16 &&
+                   ((((uintptr_t)q.x) | ((uintptr_t)q.up) | (uintptr_t)(q.x_ld * esz)) & (align - 1)) == 0;
+  load_as_f32_vec<EPL>(q.x, base, q.x_dtype, vec, nvalid, v);
+  if (q.up) load_as_f32_vec<EPL>(q.up, base, q.x_dtype, vec, nvalid, w);
 }
 
+template <int EPL>
 __device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float* v, const float* w) {
+  constexpr int UPB = 32 / EPL;
   const bool live = u.live;
   const int64_t row = u.row, kb = u.kb, k0 = u.k0;
   const int sub = u.sub;
   if (q.up) {
-    const int nvalid = q.K - k0 >= 4 ? 4 : (q.K > k0 ? (int)(q.K - k0) : 0);
-    for (int e = 0; e < 4; ++e) v[e] = (live && e < nvalid) ? silu_mul_f32(v[e], w[e]) : 0.f;
+    const int nvalid = q.K - k0 >= EPL ? EPL : (q.K > k0 ? (int)(q.K - k0) : 0);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) v[e] = (live && e < nvalid) ? silu_mul_f32(v[e], w[e]) : 0.f;
   }
   // amax over the block on |bits| (monotone in |x| for finite values; NaN patterns compare largest)
-  uint32_t bits[4], am = 0;
-  for (int e = 0; e < 4; ++e) {
+  uint32_t bits[EPL], am = 0;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
     bits[e] = __builtin_bit_cast(uint32_t, v[e]);
     const uint32_t a = bits[e] & 0x7FFFFFFFu;
     am = a > am ? a : am;
   }
-  for (int d = 1; d < 8; d <<= 1) {
+#pragma unroll
+  for (int d = 1; d < UPB; d <<= 1) {
     const uint32_t o = (uint32_t)__shfl_xor((int)am, d);
     am = o > am ? o : am;
   }
@@ -210,7 +236,7 @@ __device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float
   se = se < -127 ? -127 : (se > 127 ? 127 : se);
   const bool saturate = q.scale_mode != 0;
 
-  uint32_t code[4];
+  uint32_t code[EPL];
   // Blocks whose amax is a normal finite number and whose scale 2^se is a normal float take the hardware
   // scaled conversions (v_cvt_scalef32_pk_*: x / 2^se rounded to nearest even; FP8 overflows to NaN / inf,
   // FP4 saturates -- measured on MI355X against the integer encoders below for 270 k inputs per format).
@@ -219,69 +245,93 @@ __device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float
   if (am >= 0x00800000u && am < 0x7F800000u && se > -127 && se < 120) {
     typedef short s2 __attribute__((ext_vector_type(2)));
     const float sc = __builtin_bit_cast(float, (uint32_t)(se + 127) << 23);
-    float x[4];
-    for (int e = 0; e < 4; ++e) x[e] = v[e];
+    float x[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) x[e] = v[e];
     if (saturate && q.fmt != MX_E2M1) {
       const float lim = __fmul_rn(q.fmt == MX_E4M3 ? 448.0f : 57344.0f, sc);
-      for (int e = 0; e < 4; ++e) x[e] = __builtin_copysignf(fminf(__builtin_fabsf(x[e]), lim), x[e]);
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) x[e] = __builtin_copysignf(fminf(__builtin_fabsf(x[e]), lim), x[e]);
     }
-    uint32_t packed;
-    if (q.fmt == MX_E4M3) {
-      s2 r = {0, 0};
-      r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(r, x[0], x[1], sc, false);
-      r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(r, x[2], x[3], sc, true);
-      packed = __builtin_bit_cast(uint32_t, r);
-    } else if (q.fmt == MX_E5M2) {
-      s2 r = {0, 0};
-      r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(r, x[0], x[1], sc, false);
-      r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(r, x[2], x[3], sc, true);
-      packed = __builtin_bit_cast(uint32_t, r);
-    } else {
-      uint32_t r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, x[0], x[1], sc, 0);
-      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, x[2], x[3], sc, 1);
-      packed = (r & 0xFu) | ((r & 0xF0u) << 4) | ((r & 0xF00u) << 8) | ((r & 0xF000u) << 12);
+#pragma unroll
+    for (int h = 0; h < EPL / 4; ++h) {   // four elements at a time
+      uint32_t packed;
+      if (q.fmt == MX_E4M3) {
+        s2 r = {0, 0};
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(r, x[4 * h + 0], x[4 * h + 1], sc, false);
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(r, x[4 * h + 2], x[4 * h + 3], sc, true);
+        packed = __builtin_bit_cast(uint32_t, r);
+      } else if (q.fmt == MX_E5M2) {
+        s2 r = {0, 0};
+        r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(r, x[4 * h + 0], x[4 * h + 1], sc, false);
+        r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(r, x[4 * h + 2], x[4 * h + 3], sc, true);
+        packed = __builtin_bit_cast(uint32_t, r);
+      } else {
+        uint32_t r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, x[4 * h + 0], x[4 * h + 1], sc, 0);
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, x[4 * h + 2], x[4 * h + 3], sc, 1);
+        packed = (r & 0xFu) | ((r & 0xF0u) << 4) | ((r & 0xF00u) << 8) | ((r & 0xF000u) << 12);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) code[4 * h + e] = (packed >> (8 * e)) & 0xFFu;
     }
-    for (int e = 0; e < 4; ++e) code[e] = (packed >> (8 * e)) & 0xFFu;
   } else {
-    for (int e = 0; e < 4; ++e) {
-      const Unpacked u = unpack_f32(bits[e]);
-      code[e] = q.fmt == MX_E4M3 ? encode_e4m3(u, se, saturate)
-                : q.fmt == MX_E5M2 ? encode_e5m2(u, se, saturate)
-                                   : encode_e2m1(u, se);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      const Unpacked un = unpack_f32(bits[e]);
+      code[e] = q.fmt == MX_E4M3 ? encode_e4m3(un, se, saturate)
+                : q.fmt == MX_E5M2 ? encode_e5m2(un, se, saturate)
+                                   : encode_e2m1(un, se);
     }
   }
   if (!live) return;
   if (q.fmt == MX_E2M1) {
     // low nibble = even element (test/test_mma_scaled.py:155-160)
     uint8_t* out = q.xq + row * q.xq_ld + (k0 >> 1);
-    out[0] = (uint8_t)(code[0] | (code[1] << 4));
-    out[1] = (uint8_t)(code[2] | (code[3] << 4));
+    uint32_t word = 0;
+#pragma unroll
+    for (int e = 0; e < EPL / 2; ++e) word |= (code[2 * e] | (code[2 * e + 1] << 4)) << (8 * e);
+    if (EPL == 8 && ((((uintptr_t)q.xq) | (uintptr_t)q.xq_ld) & 3) == 0) {
+      *(uint32_t*)out = word;
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPL / 2; ++e) out[e] = (uint8_t)(word >> (8 * e));
+    }
   } else {
     uint8_t* out = q.xq + row * q.xq_ld + k0;
-    if (((((uintptr_t)q.xq) | (uintptr_t)q.xq_ld) & 3) == 0) {
-      *(uint32_t*)out = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
+    uint32_t word[EPL / 4];
+#pragma unroll
+    for (int h = 0; h < EPL / 4; ++h)
+      word[h] = code[4 * h] | (code[4 * h + 1] << 8) | (code[4 * h + 2] << 16) | (code[4 * h + 3] << 24);
+    if ((((((uintptr_t)q.xq) | (uintptr_t)q.xq_ld) & (EPL - 1))) == 0) {
+      if constexpr (EPL == 8) *(uint2*)out = make_uint2(word[0], word[1]);
+      else *(uint32_t*)out = word[0];
     } else {
-      for (int e = 0; e < 4; ++e) out[e] = (uint8_t)code[e];
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) out[e] = (uint8_t)code[e];
     }
   }
   if (sub == 0) q.scale[row * q.sc_ld + kb] = (uint8_t)(se + 127);
 }
 
-// 8 lanes per 32-element block, 4 consecutive elements per lane; every thread handles kQuantUnroll units a
-// grid apart and requests all their inputs before it processes the first (memory-level parallelism).
+// 32 / EPL lanes per 32-element block, EPL consecutive elements per lane (8: half as many threads, and the
+// per-block work -- the amax exchange, the shared exponent, the scale byte -- is spread over twice as many
+// elements; 16-byte loads also from bf16 input); every thread handles kQuantUnroll units a grid apart and
+// requests all their inputs before it processes the first (memory-level parallelism).
 constexpr int kQuantUnroll = 2;
+constexpr int kQuantEpl = 8;
+template <int EPL>
 __global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
   const int64_t nthreads = (int64_t)gridDim.x * 256;
   const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
   QuantUnit u[kQuantUnroll];
-  float v[kQuantUnroll][4], w[kQuantUnroll][4];
+  float v[kQuantUnroll][EPL], w[kQuantUnroll][EPL];
 #pragma unroll
   for (int i = 0; i < kQuantUnroll; ++i) {
-    u[i] = quant_unit(q, gid + i * nthreads);
-    quant_load(q, u[i], v[i], w[i]);
+    u[i] = quant_unit<EPL>(q, gid + i * nthreads);
+    quant_load<EPL>(q, u[i], v[i], w[i]);
   }
 #pragma unroll
-  for (int i = 0; i < kQuantUnroll; ++i) quant_store(q, u[i], v[i], w[i]);
+  for (int i = 0; i < kQuantUnroll; ++i) quant_store<EPL>(q, u[i], v[i], w[i]);
 }
 
 // ================================================================================================
@@ -539,11 +589,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 }  // namespace
 
 int launch_quantize(const QuantArgs& q, hipStream_t stream) {
-  const int64_t units = q.rows * (q.Kpad / 32) * 8;
+  const int64_t units = q.rows * (q.Kpad / 32) * (32 / kQuantEpl);
   if (units <= 0) return MX_OK;
   const int64_t blocks = (units + 256 * kQuantUnroll - 1) / (256 * kQuantUnroll);
   if (blocks > 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "quantize: tensor too large");
-  hipLaunchKernelGGL(quantize_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, q);
+  hipLaunchKernelGGL(quantize_kernel<kQuantEpl>, dim3((unsigned)blocks), dim3(256), 0, stream, q);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "quantize_kernel launch: %s", hipGetErrorString(e));
   return MX_OK;
