@@ -127,9 +127,12 @@ __device__ inline void load_as_f32_vec(const void* p, int64_t i, int dtype, bool
     }
   } else if (vec && dtype == MX_BF16) {
     uint32_t t[EPL / 2];
-    if constexpr (EPL == 8) {
-      const v4i r = *(const v4i*)((const uint16_t*)p + i);
-      t[0] = (uint32_t)r.x; t[1] = (uint32_t)r.y; t[2] = (uint32_t)r.z; t[3] = (uint32_t)r.w;
+    if constexpr (EPL >= 8) {
+#pragma unroll
+      for (int h = 0; h < EPL / 8; ++h) {
+        const v4i r = *(const v4i*)((const uint16_t*)p + i + 8 * h);
+        t[4 * h + 0] = (uint32_t)r.x; t[4 * h + 1] = (uint32_t)r.y; t[4 * h + 2] = (uint32_t)r.z; t[4 * h + 3] = (uint32_t)r.w;
+      }
     } else {
       const uint2 r = *(const uint2*)((const uint16_t*)p + i);
       t[0] = r.x; t[1] = r.y;
@@ -182,7 +185,7 @@ __device__ inline void quant_load(const QuantArgs& q, const QuantUnit& u, float*
   const int esz = q.x_dtype == MX_F32 ? 4 : 2;
   const int nvalid = q.K - u.k0 >= EPL ? EPL : (q.K > u.k0 ? (int)(q.K - u.k0) : 0);
   // 16-byte loads: fp32 in EPL / 4 pieces, bf16 as one (EPL = 8) or an 8-byte one (EPL = 4)
-  const int align = (q.x_dtype == MX_F32 || EPL == 8) ? 16 : 8;
+  const int align = (q.x_dtype == MX_F32 || EPL >= 8) ? 16 : 8;
   const bool vec = nvalid == EPL && q.x_dtype != MX_F16 &&
                    ((((uintptr_t)q.x) | ((uintptr_t)q.up) | (uintptr_t)(q.x_ld * esz)) & (align - 1)) == 0;
   load_as_f32_vec<EPL>(q.x, base, q.x_dtype, vec, nvalid, v);
@@ -287,14 +290,16 @@ __device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float
   if (q.fmt == MX_E2M1) {
     // low nibble = even element (test/test_mma_scaled.py:155-160)
     uint8_t* out = q.xq + row * q.xq_ld + (k0 >> 1);
-    uint32_t word = 0;
+    constexpr int NB = EPL / 2;   // output bytes
+    uint32_t word[(NB + 3) / 4] = {};
 #pragma unroll
-    for (int e = 0; e < EPL / 2; ++e) word |= (code[2 * e] | (code[2 * e + 1] << 4)) << (8 * e);
-    if (EPL == 8 && ((((uintptr_t)q.xq) | (uintptr_t)q.xq_ld) & 3) == 0) {
-      *(uint32_t*)out = word;
+    for (int e = 0; e < NB; ++e) word[e / 4] |= (code[2 * e] | (code[2 * e + 1] << 4)) << (8 * (e % 4));
+    if (NB >= 4 && ((((uintptr_t)q.xq) | (uintptr_t)q.xq_ld) & (NB - 1)) == 0) {
+      if constexpr (NB == 8) *(uint2*)out = make_uint2(word[0], word[1]);
+      else *(uint32_t*)out = word[0];
     } else {
 #pragma unroll
-      for (int e = 0; e < EPL / 2; ++e) out[e] = (uint8_t)(word >> (8 * e));
+      for (int e = 0; e < NB; ++e) out[e] = (uint8_t)(word[e / 4] >> (8 * (e % 4)));
     }
   } else {
     uint8_t* out = q.xq + row * q.xq_ld + k0;
@@ -303,7 +308,8 @@ __device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float
     for (int h = 0; h < EPL / 4; ++h)
       word[h] = code[4 * h] | (code[4 * h + 1] << 8) | (code[4 * h + 2] << 16) | (code[4 * h + 3] << 24);
     if ((((((uintptr_t)q.xq) | (uintptr_t)q.xq_ld) & (EPL - 1))) == 0) {
-      if constexpr (EPL == 8) *(uint2*)out = make_uint2(word[0], word[1]);
+      if constexpr (EPL == 16) *(uint4*)out = make_uint4(word[0], word[1], word[2], word[3]);
+      else if constexpr (EPL == 8) *(uint2*)out = make_uint2(word[0], word[1]);
       else *(uint32_t*)out = word[0];
     } else {
 #pragma unroll
@@ -318,7 +324,7 @@ __device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float
 // elements; 16-byte loads also from bf16 input); every thread handles kQuantUnroll units a grid apart and
 // requests all their inputs before it processes the first (memory-level parallelism).
 constexpr int kQuantUnroll = 2;
-constexpr int kQuantEpl = 8;
+constexpr int kQuantEpl = 8;    // 16 measured no faster (58 -> 60 us on 8192^2 fp32)
 template <int EPL>
 __global__ __launch_bounds__(256) void quantize_kernel(const QuantArgs q) {
   const int64_t nthreads = (int64_t)gridDim.x * 256;
