@@ -408,10 +408,18 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
   };
 
   for (int i = 0; i < t_count; ++i) {   // uniform per workgroup
-    // this wave's share of tile i has landed (its share of tile i + 1 may stay in flight) ...
+    // this wave's share of tile i has landed; its share of tile i + 1 may stay in flight, and so may the one
+    // output store that waves 0 and 1 issued after it in the previous iteration (vmcnt counts in issue order:
+    // without allowing for that store the wave would wait for the first load of tile i + 1 as well).  The
+    // count is exact only for the single-store form of the epilogue; the others wait for more than they need.
     if (i + 1 < t_count) {
-      if (with_scales) __builtin_amdgcn_s_waitcnt(0x0F70 | (Cf::WIW + 1));
-      else __builtin_amdgcn_s_waitcnt(0x0F70 | Cf::WIW);
+      const bool stored = i >= 2 && wave < 2 && vec_ok && !d.accumulate && !(VAR & 2);
+      if (with_scales) {
+        if (stored) __builtin_amdgcn_s_waitcnt(0x0F70 | (Cf::WIW + 2));
+        else __builtin_amdgcn_s_waitcnt(0x0F70 | (Cf::WIW + 1));
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | Cf::WIW);
+      }
     } else {
       __builtin_amdgcn_s_waitcnt(0x0F70);
     }
