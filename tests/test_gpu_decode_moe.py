@@ -10,7 +10,8 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("M,N,K", [(32, 256, 1024), (7, 1792, 2048), (16, 48, 512), (32, 4096, 8192), (1, 16, 4096),
-                                   (17, 4176, 4096), (29, 12320, 8192), (32, 16, 8192), (24, 36864, 4096)])
+                                   (17, 4176, 4096), (29, 12320, 8192), (32, 16, 8192), (24, 36864, 4096),
+                                   (8, 20480, 4096), (16, 16400, 8192)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=str)
 def test_decode_kernel(ct, dev, M, N, K, out_dtype):
     x = randn_operand(M, K, O.E4M3, 81, dev)
