@@ -37,8 +37,8 @@ PEAK_TFLOPS = {"mxfp8": 5033.0, "mxfp4": 10066.0}   # MI355X dense MFMA peaks (v
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the headline GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # `bench.py --only c2 --calib-copy`, each scaled by what the same counter reads for the 256 MiB copy kernel
-# (summary under profiles/): 405944 KiB x 2.0 + 135424 KiB x 1.0
-C2_HBM_TRAFFIC_BYTES = 947312 * 1024
+# (summary under profiles/): 405775 KiB x 2.0 + 132002 KiB x 1.0
+C2_HBM_TRAFFIC_BYTES = 943552 * 1024
 METRIC = "MX GEMM TFLOP/s (+% MFMA peak) 8192^3 MXFP8/MXFP4; GB/s at M=32 decode"
 
 
