@@ -23,17 +23,26 @@ SOURCES = ["mx_api.hip", "mx_gemm_mfma.hip", "mx_gemm_pp.hip", "mx_gemm_generic.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          f"-I{INCLUDE}", f"-I{CSRC}", "-Wno-unused-command-line-argument"]
-# Kernel variants with parts of the work removed (for timing studies; their results are invalid) are only
-# compiled into a library built with MXGEMM_TIMING_AIDS=1 in the environment -- never the shipped one.
-if os.environ.get("MXGEMM_TIMING_AIDS") == "1":
-    FLAGS.append("-DMXGEMM_TIMING_AIDS")
+# Extra compiler flags for experiments (for example "-DSOMETHING=1"); objects built with a different flag set
+# are never reused: the flag list is part of the up-to-date check (stamp file next to the objects).
+FLAGS += os.environ.get("MXGEMM_EXTRA_FLAGS", "").split()
 
 
 def _newer(src: pathlib.Path, obj: pathlib.Path) -> bool:
     if not obj.exists():
         return True
-    deps = [src, CSRC / "mx_common.h", CSRC / "mx_gemm_tile.h", INCLUDE / "mxgemm.h"]
+    deps = [src, *CSRC.glob("*.h"), INCLUDE / "mxgemm.h"]
     return any(d.stat().st_mtime > obj.stat().st_mtime for d in deps)
+
+
+def _flags_changed() -> bool:
+    """True (and the stamp is rewritten) when the objects on disk were built with other flags."""
+    stamp = OBJ / "flags.txt"
+    want = " ".join(FLAGS)
+    if stamp.exists() and stamp.read_text() == want:
+        return False
+    stamp.write_text(want)
+    return True
 
 
 def _compile(src: str, force: bool) -> pathlib.Path:
@@ -49,6 +58,7 @@ def _compile(src: str, force: bool) -> pathlib.Path:
 
 def build(force: bool = False, jobs: int | None = None) -> pathlib.Path:
     OBJ.mkdir(exist_ok=True)
+    force = _flags_changed() or force
     jobs = jobs or min(len(SOURCES), os.cpu_count() or 4, 8)
     with ThreadPoolExecutor(jobs) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), SOURCES))

@@ -23,12 +23,8 @@ namespace {
 inline bool is_elem(int d) { return d == MX_E4M3 || d == MX_E5M2 || d == MX_E2M1; }
 inline int64_t round256(int64_t b) { return (b + 255) & ~(int64_t)255; }
 
-// kernel MX_KERNEL_AUTO uses for large problems; MXGEMM_PP=0 (read once) selects the non-ping-pong
-// 256x256 kernel instead, for side-by-side timing
-int big_tile_kernel() {
-  static const int pp = [] { const char* e = getenv("MXGEMM_PP"); return e ? atoi(e) : 1; }();
-  return pp ? MX_KERNEL_MFMA_PINGPONG : MX_KERNEL_MFMA_256x256;
-}
+// kernel MX_KERNEL_AUTO uses for large problems
+constexpr int big_tile_kernel() { return MX_KERNEL_MFMA_PINGPONG; }
 
 // Problems MX_KERNEL_AUTO gives to the persistent 256x256 kernel: enough 256x256 tiles to occupy most of the
 // 256 CUs (measured crossover against the 128x128 one-tile kernel, which has four times as many workgroups
@@ -144,6 +140,19 @@ int64_t mx_gemm_grouped_workspace_bytes(int64_t num_slots, int64_t N, int64_t K,
 }
 
 namespace {
+// a 4-D swizzle_32_4_4 scale tensor must be the contiguous [rows / 128, (K / 32) / 4, 32, 16] array
+int check_swizzled_scale(const mx_tensor* scale, const char* name, int64_t rows, int64_t KB) {
+  if (scale->ndim != 4 || scale->shape[2] != 32 || scale->shape[3] != 16)
+    return set_error(MX_ERR_SHAPE, "%s: swizzled scale layout expects [rows/128, K/128, 32, 16]", name);
+  if (rows % 128 != 0 || KB % 4 != 0 || scale->shape[0] != rows / 128 || scale->shape[1] != KB / 4)
+    return set_error(MX_ERR_SHAPE, "%s: swizzled scale shape does not match rows=%lld, K blocks=%lld (rows %% 128 "
+                     "and blocks %% 4 must be 0)", name, (long long)rows, (long long)KB);
+  if (scale->stride[3] != 1 || scale->stride[2] != 16 || scale->stride[1] != 512 ||
+      scale->stride[0] != 512 * (KB / 4))
+    return set_error(MX_ERR_LAYOUT, "%s: swizzled scale tensor must be contiguous", name);
+  return MX_OK;
+}
+
 // validates a scale tensor against (rows, K) and describes its re-layout into `packed`
 int make_pack_args(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, void* packed, PackArgs& p) {
   if (int rc = check_tensor(scale, "scale", 2, 4)) return rc;
@@ -173,14 +182,7 @@ int make_pack_args(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t
       p.s_batch = scale->stride[0];
     }
   } else if (layout == MX_SCALE_SWIZZLE_32_4_4) {
-    if (scale->ndim != 4 || scale->shape[2] != 32 || scale->shape[3] != 16)
-      return set_error(MX_ERR_SHAPE, "swizzled scale layout expects [rows/128, K/128, 32, 16]");
-    if (rows % 128 != 0 || KB % 4 != 0 || scale->shape[0] != rows / 128 || scale->shape[1] != KB / 4)
-      return set_error(MX_ERR_SHAPE, "swizzled scale shape does not match rows=%lld, K=%lld", (long long)rows,
-                       (long long)K);
-    if (scale->stride[3] != 1 || scale->stride[2] != 16 || scale->stride[1] != 512 ||
-        scale->stride[0] != 512 * (KB / 4))
-      return set_error(MX_ERR_LAYOUT, "swizzled scale tensor must be contiguous");
+    if (int rc = check_swizzled_scale(scale, "scale", rows, KB)) return rc;
   } else {
     return set_error(MX_ERR_INVALID, "mx_pack_scales: unknown source layout %d", layout);
   }
@@ -314,6 +316,14 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
       return set_error(MX_ERR_DTYPE, "E4M3 scales are only defined for FP4 operands with block size 16");
     if (o.block_size == 16 && (A->dtype != MX_E2M1 || B->dtype != MX_E2M1))
       return set_error(MX_ERR_DTYPE, "block size 16 is only defined for FP4 operands");
+    if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF || batch > 0x7FFFFFFF)
+      return set_error(MX_ERR_SHAPE, "extents of 2^31 or more are not supported");
+    if ((o.a_scale_layout == MX_SCALE_SWIZZLE_32_4_4 || o.b_scale_layout == MX_SCALE_SWIZZLE_32_4_4) && batched)
+      return set_error(MX_ERR_LAYOUT, "swizzled scale tensors have no batch dimension");
+    if (o.a_scale_layout == MX_SCALE_SWIZZLE_32_4_4)
+      if (int rc = check_swizzled_scale(As, "A_scale", M, KB)) return rc;
+    if (o.b_scale_layout == MX_SCALE_SWIZZLE_32_4_4)
+      if (int rc = check_swizzled_scale(Bs, "B_scale", N, KB)) return rc;
     GenericArgs g = {};
     g.A = (const uint8_t*)A->ptr; g.As = (const uint8_t*)As->ptr;
     g.B = (const uint8_t*)B->ptr; g.Bs = (const uint8_t*)Bs->ptr; g.C = C->ptr;
@@ -330,15 +340,11 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
       const int nd = As->ndim;
       g.as_sb = (nd == 3 && batchA > 1) ? As->stride[0] : 0;
       g.as_sm = As->stride[nd - 2]; g.as_sk = As->stride[nd - 1];
-    } else if (M % 128 != 0 || KB % 4 != 0) {
-      return set_error(MX_ERR_SHAPE, "swizzled A_scale needs M %% 128 == 0 and (K/32) %% 4 == 0");
     }
     if (o.b_scale_layout == MX_SCALE_2D) {
       const int nd = Bs->ndim;
       g.bs_sb = (nd == 3 && batchB > 1) ? Bs->stride[0] : 0;
       g.bs_sk = Bs->stride[nd - 2]; g.bs_sn = Bs->stride[nd - 1];
-    } else if (N % 128 != 0 || KB % 4 != 0) {
-      return set_error(MX_ERR_SHAPE, "swizzled B_scale needs N %% 128 == 0 and (K/32) %% 4 == 0");
     }
     g.c_sb = cnd == 3 ? C->stride[0] : 0; g.c_sm = C->stride[cnd - 2]; g.c_sn = C->stride[cnd - 1];
     return launch_gemm_generic(g, (hipStream_t)stream);
@@ -482,6 +488,40 @@ int mx_gemm_list(int32_t count, const mx_tensor* A, const mx_tensor* As, const m
   return MX_OK;
 }
 
+int mx_bench_gemm(int32_t nsets, const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const mx_tensor* Bs,
+                  mx_tensor* C, const mx_gemm_opts* opts, void* workspace, int64_t workspace_bytes, int32_t warmup,
+                  int32_t iters, float* times_ms, void* stream) {
+  if (nsets <= 0 || !A || !As || !B || !Bs || !C) return set_error(MX_ERR_INVALID, "mx_bench_gemm: no operand sets");
+  if (warmup < 0 || iters <= 0 || iters > 65536 || !times_ms)
+    return set_error(MX_ERR_INVALID, "mx_bench_gemm: iters must be in 1..65536 and times_ms non-null");
+  hipStream_t st = (hipStream_t)stream;
+  for (int i = 0; i < warmup; ++i) {
+    const int s = i % nsets;
+    if (int rc = mx_gemm(&A[s], &As[s], &B[s], &Bs[s], &C[s], opts, workspace, workspace_bytes, stream)) return rc;
+  }
+  hipEvent_t* ev = (hipEvent_t*)calloc((size_t)2 * iters, sizeof(hipEvent_t));
+  if (!ev) return set_error(MX_ERR_INVALID, "mx_bench_gemm: out of host memory");
+  int rc = MX_OK, made = 0;
+  for (; made < 2 * iters; ++made)
+    if (hipEventCreate(&ev[made]) != hipSuccess) { rc = set_error(MX_ERR_DEVICE, "mx_bench_gemm: hipEventCreate failed"); break; }
+  for (int i = 0; rc == MX_OK && i < iters; ++i) {
+    const int s = (warmup + i) % nsets;
+    if (hipEventRecord(ev[2 * i], st) != hipSuccess) { rc = set_error(MX_ERR_DEVICE, "mx_bench_gemm: hipEventRecord failed"); break; }
+    rc = mx_gemm(&A[s], &As[s], &B[s], &Bs[s], &C[s], opts, workspace, workspace_bytes, stream);
+    if (rc == MX_OK && hipEventRecord(ev[2 * i + 1], st) != hipSuccess)
+      rc = set_error(MX_ERR_DEVICE, "mx_bench_gemm: hipEventRecord failed");
+  }
+  // the stream is drained on every path, so that no event is destroyed while still pending
+  const hipError_t es = hipStreamSynchronize(st);
+  if (rc == MX_OK && es != hipSuccess) rc = set_error(MX_ERR_DEVICE, "mx_bench_gemm: %s", hipGetErrorString(es));
+  for (int i = 0; rc == MX_OK && i < iters; ++i)
+    if (hipEventElapsedTime(&times_ms[i], ev[2 * i], ev[2 * i + 1]) != hipSuccess)
+      rc = set_error(MX_ERR_DEVICE, "mx_bench_gemm: hipEventElapsedTime failed");
+  for (int i = 0; i < made; ++i) (void)hipEventDestroy(ev[i]);
+  free(ev);
+  return rc;
+}
+
 int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W, const mx_tensor* Ws,
                     mx_tensor* C, const float* topk_weights, const int32_t* sorted_token_ids,
                     int64_t num_slots, const int32_t* sorted_expert_ids, int32_t tile_m,
@@ -598,17 +638,29 @@ int64_t mx_moe_align_max_slots(int64_t num_ids, int32_t num_experts, int32_t til
   return (num_ids + nonempty * (tile_m - 1)) / tile_m * tile_m;
 }
 
+int64_t mx_moe_align_workspace_bytes(int64_t num_ids, int32_t num_experts) {
+  if (num_ids <= 0 || num_experts <= 0) return 0;
+  return round256(moe_align_workspace_bytes(num_ids, num_experts));
+}
+
 int mx_moe_align(const int32_t* topk_ids, int64_t num_ids, int32_t num_experts, int32_t tile_m,
-                 int32_t* sorted_token_ids, int32_t* sorted_expert_ids, int32_t* num_slots_out, void* stream) {
+                 int32_t* sorted_token_ids, int32_t* sorted_expert_ids, int32_t* num_slots_out, void* workspace,
+                 int64_t workspace_bytes, void* stream) {
   if (num_ids < 0 || num_experts <= 0 || tile_m <= 0) return set_error(MX_ERR_INVALID, "moe_align: bad sizes");
   if (num_ids >= 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "moe_align: too many ids");
   const int64_t max_slots = mx_moe_align_max_slots(num_ids, num_experts, tile_m);
   if (max_slots == 0) {
     return MX_OK;
   }
+  if (max_slots >= 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "moe_align: too many slots");
   if (!topk_ids || !sorted_token_ids || !sorted_expert_ids) return set_error(MX_ERR_INVALID, "moe_align: null pointer");
+  const int64_t need = moe_align_workspace_bytes(num_ids, num_experts);
+  if (need > 0 && (!workspace || workspace_bytes < need))
+    return set_error(MX_ERR_WORKSPACE, "moe_align: workspace of %lld bytes required, %lld given", (long long)need,
+                     (long long)workspace_bytes);
+  if (need > 0 && ((uintptr_t)workspace) % 4 != 0) return set_error(MX_ERR_WORKSPACE, "moe_align: workspace must be 4-byte aligned");
   return launch_moe_align(topk_ids, num_ids, num_experts, tile_m, sorted_token_ids, sorted_expert_ids,
-                          num_slots_out, max_slots, (hipStream_t)stream);
+                          num_slots_out, max_slots, (int32_t*)workspace, (hipStream_t)stream);
 }
 
 namespace {

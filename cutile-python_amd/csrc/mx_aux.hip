@@ -221,8 +221,9 @@ __device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float
   int se;
   if (q.scale_mode == 0) {
     // reference rule: 2^ceil(log2(max(amax/448, 1e-12))), ceiling taken exactly on the fp32 quotient
+    // (a block with an inf or NaN amax never uses this exponent: see nonfinite_ceil below)
     float t = __fdiv_rn(__builtin_bit_cast(float, am), 448.0f);
-    t = t > 1e-12f ? t : 1e-12f;              // NaN compares false -> 1e-12, as torch.clamp(min=) does not; see below
+    t = t > 1e-12f ? t : 1e-12f;
     const uint32_t tb = __builtin_bit_cast(uint32_t, t);
     se = (int)(tb >> 23) - 127 + ((tb & 0x7FFFFFu) ? 1 : 0);
   } else {
@@ -239,7 +240,25 @@ __device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float
   se = se < -127 ? -127 : (se > 127 ? 127 : se);
   const bool saturate = q.scale_mode != 0;
 
+  // Reference rule with a non-finite amax: torch.clamp(min=) keeps NaN and inf / 448 stays inf, so the scale is
+  // NaN or inf, both of which the cast to float8_e8m0fnu writes as 0xFF; x / scale is then NaN for every
+  // element of a NaN block (the element's own sign if it is a NaN itself), and for an inf block NaN where
+  // |x| is inf (inf / inf is the default NaN, whose sign bit is set on the hosts the reference runs on) and a
+  // signed zero elsewhere.  E2M1 has no NaN: non-finite elements saturate to +-6 as in the finite case.
+  const bool nonfinite_ceil = q.scale_mode == 0 && am >= 0x7F800000u;
   uint32_t code[EPL];
+  if (nonfinite_ceil) {
+    const bool blk_nan = am > 0x7F800000u;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      const uint32_t a = bits[e] & 0x7FFFFFFFu, sgn = bits[e] >> 31;
+      if (q.fmt == MX_E2M1) code[e] = (sgn << 3) | ((blk_nan || a == 0x7F800000u) ? 7u : 0u);
+      else if (a > 0x7F800000u) code[e] = (sgn << 7) | 0x7Fu;
+      else if (blk_nan) code[e] = 0x7Fu;
+      else if (a == 0x7F800000u) code[e] = 0xFFu;
+      else code[e] = sgn << 7;
+    }
+  } else
   // Blocks whose amax is a normal finite number and whose scale 2^se is a normal float take the hardware
   // scaled conversions (v_cvt_scalef32_pk_*: x / 2^se rounded to nearest even; FP8 overflows to NaN / inf,
   // FP4 saturates -- measured on MI355X against the integer encoders below for 270 k inputs per format).
@@ -316,7 +335,7 @@ __device__ inline void quant_store(const QuantArgs& q, const QuantUnit& u, float
       for (int e = 0; e < EPL; ++e) out[e] = (uint8_t)code[e];
     }
   }
-  if (sub == 0) q.scale[row * q.sc_ld + kb] = (uint8_t)(se + 127);
+  if (sub == 0) q.scale[row * q.sc_ld + kb] = nonfinite_ceil ? (uint8_t)0xFF : (uint8_t)(se + 127);
 }
 
 // 32 / EPL lanes per 32-element block, EPL consecutive elements per lane (8: half as many threads, and the
@@ -428,137 +447,175 @@ __global__ __launch_bounds__(256) void pack_scales_kernel(const PackPair pp) {
 // ================================================================================================
 // MoE slot alignment (replaces moe_align_tile_size_torch, test/kernels/fused_moe.py:113-173)
 // ================================================================================================
-// One workgroup.  Phase 1: histogram of expert ids.  Phase 2: exclusive scan of the per-expert block
-// counts.  Phase 3: wave 0 walks the ids in order, 64 at a time, and places each at
-// start[expert] + (number of earlier ids of that expert): a stable counting sort.
-__global__ __launch_bounds__(256) void moe_align_kernel(const int32_t* __restrict__ topk_ids, int64_t n,
-                                                        int32_t E, int32_t tile_m,
-                                                        int32_t* __restrict__ sorted_ids,
-                                                        int32_t* __restrict__ expert_ids,
-                                                        int32_t* __restrict__ num_slots_out,
-                                                        int64_t max_slots) {
-  extern __shared__ int32_t sh[];
-  int32_t* cnt = sh;          // [E] counts, then running write cursor
-  int32_t* start = sh + E;    // [E + 1] first slot of each expert
+// A stable counting sort of the flattened expert ids over several workgroups, without atomics on global
+// memory and without any slot written twice.  The ids are cut into B contiguous chunks, one per workgroup.
+//   moe_hist_kernel (only when B > 1): workgroup b counts the ids of every expert in chunk b -> counts[b][e].
+//   moe_place_kernel: workgroup b
+//     1. sums column e of `counts` (thread e): ids of expert e in all chunks (total) and in the chunks before
+//        its own (base); with B == 1 the totals come from its own counting pass instead;
+//     2. exclusive scan of the tile-padded totals over the experts -> first slot of every expert (start);
+//     3. places the ids of its chunk in order at start[e] + base[e] + (rank inside the chunk).  Up to 256
+//        experts: every thread owns a contiguous segment of the chunk, per-thread per-expert counts live in
+//        LDS as u16 (a chunk holds at most 65535 ids, so neither a count nor a prefix inside the chunk can
+//        wrap) and become exclusive prefixes over the threads, which is what makes the order stable; more
+//        experts: wave 0 walks the chunk 64 ids at a time and ranks equal experts with ballots;
+//     4. experts b, b + B, ... : sentinel into the padding behind the expert's ids, expert id into its blocks;
+//        all workgroups together: sentinel / expert 0 into the unused tail of the worst-case-sized outputs.
+constexpr int kAlignThreads = 256;
+constexpr int kAlignSegExperts = 256;      // up to this many experts the segment placement is used
+constexpr int64_t kAlignMaxChunk = 65535;  // ids per workgroup (u16 prefixes inside a chunk)
+
+__global__ __launch_bounds__(kAlignThreads) void moe_hist_kernel(const int32_t* __restrict__ topk_ids, int64_t n,
+                                                                 int32_t E, int64_t chunk,
+                                                                 int32_t* __restrict__ counts) {
+  extern __shared__ int32_t sh[];   // [E]
   const int tid = threadIdx.x;
-  for (int e = tid; e < E; e += 256) cnt[e] = 0;
-  for (int64_t i = tid; i < max_slots; i += 256) sorted_ids[i] = (int32_t)n;
+  for (int e = tid; e < E; e += kAlignThreads) sh[e] = 0;
   __syncthreads();
-  for (int64_t i = tid; i < n; i += 256) {
+  const int64_t lo = (int64_t)blockIdx.x * chunk, hi = lo + chunk < n ? lo + chunk : n;
+  for (int64_t i = lo + tid; i < hi; i += kAlignThreads) {
     const int e = topk_ids[i];
-    if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+    if (e >= 0 && e < E) atomicAdd(&sh[e], 1);
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += kAlignThreads) counts[(int64_t)blockIdx.x * E + e] = sh[e];
+}
+
+__global__ __launch_bounds__(kAlignThreads) void moe_place_kernel(const int32_t* __restrict__ topk_ids, int64_t n,
+                                                                  int32_t E, int32_t tile_m, int64_t chunk,
+                                                                  const int32_t* __restrict__ counts,
+                                                                  int32_t* __restrict__ sorted_ids,
+                                                                  int32_t* __restrict__ expert_ids,
+                                                                  int32_t* __restrict__ num_slots_out,
+                                                                  int64_t max_slots) {
+  constexpr int T = kAlignThreads, LD = T + 2;   // row pitch 129 dwords: rows start on consecutive LDS banks
+  extern __shared__ int32_t sh[];
+  int32_t* total = sh;                  // [E] ids per expert
+  int32_t* base = sh + E;               // [E] ids of the expert in earlier chunks; later the write cursor
+  int32_t* start = sh + 2 * E;          // [E + 1] first slot of each expert
+  int32_t* part = sh + 3 * E + 1;       // [T] partial sums of the scan
+  uint16_t* cnt = (uint16_t*)(sh + 3 * E + 1 + T);   // [E][LD], segment placement only
+  const int tid = threadIdx.x, B = gridDim.x, b = blockIdx.x;
+  const bool seg_mode = E <= kAlignSegExperts;
+  const int64_t lo = (int64_t)b * chunk, hi = lo + chunk < n ? lo + chunk : n;
+  const int64_t seg = (hi - lo + T - 1) / T;
+  const int64_t slo = lo + tid * seg < hi ? lo + tid * seg : hi, shi = slo + seg < hi ? slo + seg : hi;
+
+  // ---- 1. totals and bases ------------------------------------------------------------------------------
+  if (seg_mode) {
+    for (int i = tid; i < E * LD / 2; i += T) ((uint32_t*)cnt)[i] = 0;
+    __syncthreads();
+    for (int64_t i = slo; i < shi; ++i) {
+      const int e = topk_ids[i];
+      if (e >= 0 && e < E) cnt[e * LD + tid] += 1;
+    }
+    __syncthreads();
+    if (tid < E) {   // row e -> exclusive prefixes over the threads; the row sum is the chunk's count
+      uint16_t* row = cnt + tid * LD;
+      int32_t run = 0;
+      for (int t = 0; t < T; ++t) {
+        const int32_t c = row[t];
+        row[t] = (uint16_t)run;
+        run += c;
+      }
+      total[tid] = run;
+    }
+  } else if (B == 1) {
+    for (int e = tid; e < E; e += T) total[e] = 0;
+    __syncthreads();
+    for (int64_t i = lo + tid; i < hi; i += T) {
+      const int e = topk_ids[i];
+      if (e >= 0 && e < E) atomicAdd(&total[e], 1);
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += T) {
+    int32_t pre = 0;
+    if (B > 1) {
+      int32_t tot = 0;
+      for (int bb = 0; bb < B; ++bb) {
+        const int32_t c = counts[(int64_t)bb * E + e];
+        if (bb < b) pre += c;
+        tot += c;
+      }
+      total[e] = tot;
+    }
+    base[e] = pre;
+  }
+  __syncthreads();
+  // ---- 2. first slot of every expert: thread t scans experts [t * per, (t + 1) * per) -------------------
+  const int per = (E + T - 1) / T;
+  {
+    int32_t s2 = 0;
+    for (int e = tid * per; e < (tid + 1) * per && e < E; ++e) s2 += (total[e] + tile_m - 1) / tile_m * tile_m;
+    part[tid] = s2;
   }
   __syncthreads();
   if (tid == 0) {
-    int32_t s = 0;
-    for (int e = 0; e < E; ++e) {
-      start[e] = s;
-      s += (cnt[e] + tile_m - 1) / tile_m * tile_m;
+    int32_t run = 0;
+    for (int t = 0; t < T; ++t) {
+      const int32_t c = part[t];
+      part[t] = run;
+      run += c;
     }
-    start[E] = s;
-    if (num_slots_out) *num_slots_out = s;
+    start[E] = run;
+    if (b == 0 && num_slots_out) *num_slots_out = run;
   }
   __syncthreads();
-  // block -> expert map; trailing unused blocks name expert 0 (their slots hold the sentinel)
-  const int64_t max_blocks = max_slots / tile_m;
-  for (int64_t blk = tid; blk < max_blocks; blk += 256) expert_ids[blk] = 0;
-  __syncthreads();
-  for (int e = tid; e < E; e += 256) {
-    for (int32_t s = start[e]; s < start[e + 1]; s += tile_m) expert_ids[s / tile_m] = e;
-    cnt[e] = start[e];  // becomes the write cursor
+  {
+    int32_t run = part[tid];
+    for (int e = tid * per; e < (tid + 1) * per && e < E; ++e) {
+      start[e] = run;
+      run += (total[e] + tile_m - 1) / tile_m * tile_m;
+    }
   }
   __syncthreads();
-  if (tid < 64) {
-    for (int64_t base = 0; base < n; base += 64) {
-      const int64_t i = base + tid;
-      int e = i < n ? topk_ids[i] : -1;
-      if (e >= E) e = -1;
-      bool todo = e >= 0;
-      while (__any(todo)) {
-        const uint64_t pending = __ballot(todo);
-        const int leader = __builtin_ctzll(pending);
-        const int e0 = __shfl(e, leader);
-        const bool mine = todo && e == e0;
-        const uint64_t same = __ballot(mine);
-        if (mine) {
-          const int rank = __builtin_popcountll(same & ((1ull << tid) - 1ull));
-          sorted_ids[cnt[e0] + rank] = (int32_t)i;
-          todo = false;
+  // ---- 3. placement -------------------------------------------------------------------------------------
+  if (seg_mode) {
+    for (int64_t i = slo; i < shi; ++i) {
+      const int e = topk_ids[i];
+      if (e >= 0 && e < E) {
+        const int32_t pos = start[e] + base[e] + cnt[e * LD + tid];
+        cnt[e * LD + tid] += 1;
+        sorted_ids[pos] = (int32_t)i;
+      }
+    }
+  } else {
+    for (int e = tid; e < E; e += T) base[e] += start[e];   // write cursor of this chunk
+    __syncthreads();
+    if (tid < 64) {
+      for (int64_t i0 = lo; i0 < hi; i0 += 64) {
+        const int64_t i = i0 + tid;
+        int e = i < hi ? topk_ids[i] : -1;
+        if (e >= E) e = -1;
+        bool todo = e >= 0;
+        while (__any(todo)) {
+          const uint64_t pending = __ballot(todo);
+          const int leader = __builtin_ctzll(pending);
+          const int e0 = __shfl(e, leader);
+          const bool mine = todo && e == e0;
+          const uint64_t same = __ballot(mine);
+          if (mine) {
+            const int rank = __builtin_popcountll(same & ((1ull << tid) - 1ull));
+            sorted_ids[base[e0] + rank] = (int32_t)i;
+            todo = false;
+          }
+          if (tid == leader) base[e0] += __builtin_popcountll(same);
+          // wave-synchronous: the next iteration's reads of base[] follow this write in program order
+          __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
         }
-        if (tid == leader) cnt[e0] += __builtin_popcountll(same);
-        // wave-synchronous: the next iteration's reads of cnt[] follow this write in program order
-        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
       }
     }
   }
-}
-
-// Parallel variant for E <= 256 experts: every thread owns a contiguous segment of the ids.
-//   1. per-thread, per-expert counts (LDS, u16, one column per thread: no atomics);
-//   2. thread e turns row e into exclusive prefixes over the threads (earlier segments come first, which is
-//      what makes the sort stable) and keeps the expert's total;
-//   3. exclusive scan of the tile-padded totals over the experts;
-//   4. every thread places its segment in order at start[e] + prefix[e][thread]++;
-//   5. padding slots get the sentinel n, blocks get their expert.  No slot is written twice.
-__global__ __launch_bounds__(256) void moe_align_seg_kernel(const int32_t* __restrict__ topk_ids, int64_t n,
-                                                            int32_t E, int32_t tile_m,
-                                                            int32_t* __restrict__ sorted_ids,
-                                                            int32_t* __restrict__ expert_ids,
-                                                            int32_t* __restrict__ num_slots_out,
-                                                            int64_t max_slots) {
-  constexpr int T = 256, LD = T + 2;   // row pitch 129 dwords: rows start on consecutive LDS banks
-  extern __shared__ int32_t sh[];
-  int32_t* total = sh;                  // [E] ids per expert
-  int32_t* start = sh + E;              // [E + 1] first slot of each expert
-  uint16_t* cnt = (uint16_t*)(sh + 2 * E + 2);   // [E][LD]
-  const int tid = threadIdx.x;
-  const int64_t seg = (n + T - 1) / T;
-  const int64_t lo = tid * seg < n ? tid * seg : n, hi = lo + seg < n ? lo + seg : n;
-  for (int i = tid; i < E * LD / 2; i += T) ((uint32_t*)cnt)[i] = 0;
-  __syncthreads();
-  for (int64_t i = lo; i < hi; ++i) {
-    const int e = topk_ids[i];
-    if (e >= 0 && e < E) cnt[e * LD + tid] += 1;
-  }
-  __syncthreads();
-  if (tid < E) {
-    uint16_t* row = cnt + tid * LD;
-    int32_t run = 0;
-    for (int t = 0; t < T; ++t) {
-      const int32_t c = row[t];
-      row[t] = (uint16_t)run;
-      run += c;
-    }
-    total[tid] = run;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    int32_t s = 0;
-    for (int e = 0; e < E; ++e) {
-      start[e] = s;
-      s += (total[e] + tile_m - 1) / tile_m * tile_m;
-    }
-    start[E] = s;
-    if (num_slots_out) *num_slots_out = s;
-  }
-  __syncthreads();
-  for (int64_t i = lo; i < hi; ++i) {
-    const int e = topk_ids[i];
-    if (e >= 0 && e < E) {
-      const int32_t pos = start[e] + cnt[e * LD + tid];
-      cnt[e * LD + tid] += 1;
-      sorted_ids[pos] = (int32_t)i;
-    }
-  }
-  // padding behind every expert's ids, the unused tail, and the block -> expert map (trailing unused
-  // blocks name expert 0; their slots hold the sentinel)
-  for (int e = tid; e < E; e += T) {
-    for (int32_t s2 = start[e] + total[e]; s2 < start[e + 1]; ++s2) sorted_ids[s2] = (int32_t)n;
-    for (int32_t s2 = start[e]; s2 < start[e + 1]; s2 += tile_m) expert_ids[s2 / tile_m] = e;
+  // ---- 4. padding, block -> expert map, unused tail (trailing blocks name expert 0) -------------------------
+  for (int e = b; e < E; e += B) {
+    for (int32_t s2 = start[e] + total[e] + tid; s2 < start[e + 1]; s2 += T) sorted_ids[s2] = (int32_t)n;
+    for (int32_t s2 = start[e] + tid * tile_m; s2 < start[e + 1]; s2 += T * tile_m) expert_ids[s2 / tile_m] = e;
   }
   const int32_t used = start[E];
-  for (int64_t i = used + tid; i < max_slots; i += T) sorted_ids[i] = (int32_t)n;
-  for (int64_t blk = used / tile_m + tid; blk < max_slots / tile_m; blk += T) expert_ids[blk] = 0;
+  for (int64_t i = used + (int64_t)b * T + tid; i < max_slots; i += (int64_t)B * T) sorted_ids[i] = (int32_t)n;
+  for (int64_t blk = used / tile_m + (int64_t)b * T + tid; blk < max_slots / tile_m; blk += (int64_t)B * T)
+    expert_ids[blk] = 0;
 }
 
 // ================================================================================================
@@ -642,28 +699,48 @@ int launch_splitk_reduce(const float* partials, int splits, int64_t M, int64_t N
   return MX_OK;
 }
 
+// chunks (= workgroups) the ids are cut into: about 1024 ids each, at most 256 chunks unless a chunk would then
+// exceed what the u16 prefixes of the placement hold
+void moe_align_plan(int64_t num_ids, int64_t& chunk, int64_t& blocks) {
+  chunk = (num_ids + 255) / 256;
+  if (chunk < 1024) chunk = 1024;
+  if (chunk > kAlignMaxChunk) chunk = kAlignMaxChunk;
+  blocks = num_ids > 0 ? (num_ids + chunk - 1) / chunk : 1;
+}
+
+int64_t moe_align_workspace_bytes(int64_t num_ids, int32_t num_experts) {
+  int64_t chunk, blocks;
+  moe_align_plan(num_ids, chunk, blocks);
+  return blocks > 1 ? blocks * num_experts * (int64_t)sizeof(int32_t) : 0;
+}
+
 int launch_moe_align(const int32_t* topk_ids, int64_t num_ids, int32_t num_experts, int32_t tile_m,
                      int32_t* sorted_token_ids, int32_t* sorted_expert_ids, int32_t* num_slots_out,
-                     int64_t max_slots, hipStream_t stream) {
-  if (num_experts <= 256 && num_ids <= (int64_t)256 * 65535) {
-    const size_t lds = (size_t)(2 * num_experts + 2) * sizeof(int32_t) + (size_t)num_experts * 258 * sizeof(uint16_t);
-    static int attr_done = 0;   // benign race: the attribute call is idempotent
-    if (!attr_done) {
-      hipError_t e = hipFuncSetAttribute((const void*)moe_align_seg_kernel,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-      if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "hipFuncSetAttribute(moe_align): %s", hipGetErrorString(e));
-      attr_done = 1;
-    }
-    hipLaunchKernelGGL(moe_align_seg_kernel, dim3(1), dim3(256), lds, stream, topk_ids, num_ids, num_experts,
-                       tile_m, sorted_token_ids, sorted_expert_ids, num_slots_out, max_slots);
-  } else {
-    const size_t lds = (size_t)(2 * num_experts + 1) * sizeof(int32_t);
-    if (lds > 60000) return set_error(MX_ERR_SHAPE, "moe_align: too many experts (%d)", num_experts);
-    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(256), lds, stream, topk_ids, num_ids, num_experts,
-                       tile_m, sorted_token_ids, sorted_expert_ids, num_slots_out, max_slots);
+                     int64_t max_slots, int32_t* counts, hipStream_t stream) {
+  int64_t chunk, blocks;
+  moe_align_plan(num_ids, chunk, blocks);
+  const bool seg = num_experts <= kAlignSegExperts;
+  const size_t lds = (size_t)(3 * num_experts + 1 + kAlignThreads) * sizeof(int32_t) +
+                     (seg ? (size_t)num_experts * (kAlignThreads + 2) * sizeof(uint16_t) : 0);
+  if (lds > 150 * 1024) return set_error(MX_ERR_SHAPE, "moe_align: too many experts (%d)", num_experts);
+  if (blocks > 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "moe_align: too many ids");
+  static int attr_done = 0;   // benign race: the attribute call is idempotent
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void*)moe_place_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       160 * 1024);
+    if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "hipFuncSetAttribute(moe_align): %s", hipGetErrorString(e));
+    attr_done = 1;
   }
+  if (blocks > 1) {
+    hipLaunchKernelGGL(moe_hist_kernel, dim3((unsigned)blocks), dim3(kAlignThreads), (size_t)num_experts * sizeof(int32_t),
+                       stream, topk_ids, num_ids, num_experts, chunk, counts);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "moe_hist_kernel launch: %s", hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(moe_place_kernel, dim3((unsigned)blocks), dim3(kAlignThreads), lds, stream, topk_ids, num_ids,
+                     num_experts, tile_m, chunk, counts, sorted_token_ids, sorted_expert_ids, num_slots_out, max_slots);
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "moe_align_kernel launch: %s", hipGetErrorString(e));
+  if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "moe_place_kernel launch: %s", hipGetErrorString(e));
   return MX_OK;
 }
 

@@ -149,9 +149,11 @@ struct QuantArgs {
 };
 int launch_quantize(const QuantArgs& q, hipStream_t stream);
 
+// `counts`: moe_align_workspace_bytes(num_ids, num_experts) bytes of scratch (per-chunk histograms)
+int64_t moe_align_workspace_bytes(int64_t num_ids, int32_t num_experts);
 int launch_moe_align(const int32_t* topk_ids, int64_t num_ids, int32_t num_experts, int32_t tile_m,
                      int32_t* sorted_token_ids, int32_t* sorted_expert_ids, int32_t* num_slots_out,
-                     int64_t max_slots, hipStream_t stream);
+                     int64_t max_slots, int32_t* counts, hipStream_t stream);
 
 struct DecodeArgs {
   const uint8_t* X; const uint8_t* Xs; const uint8_t* W; const uint8_t* Ws; void* C;

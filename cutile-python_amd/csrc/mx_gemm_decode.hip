@@ -61,7 +61,7 @@ __device__ inline void issue_tile_dma(const uint8_t* W, uint32_t wbytes, const u
   __builtin_amdgcn_raw_ptr_buffer_load_lds(rsS, (lds_void*)(base + SPW * 1024), 16, soff, ssoff, 0, 0);
 }
 
-template <int XF, int SPW, int MT, typename OutT, int VAR = 0>
+template <int XF, int SPW, int MT, typename OutT>
 __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d) {
   using Cf = DecodeCfg<SPW, MT>;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
@@ -114,7 +114,6 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
       const int ks = s0 + s < ksteps ? s0 + s : 0;
-      if constexpr ((VAR & 4) != 0) { xlo[i][s] = (v4i){s, 1, 2, 3}; xhi[i][s] = xlo[i][s]; continue; }
       xlo[i][s] = *(const v4i*)(xrow + (int64_t)ks * 128);
       xhi[i][s] = *(const v4i*)(xrow + (int64_t)ks * 128 + 64);
     }
@@ -183,7 +182,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
 #pragma unroll
         for (int h = 0; h < Cf::SB / 16; ++h) sc[h] = *(lds_cv4i*)(st + r * Cf::SB + 16 * h);
 #pragma unroll
-        for (int s = 0; s < ((VAR & 1) ? 0 : SPW); ++s) {
+        for (int s = 0; s < SPW; ++s) {
           const v4i w = *(lds_cv4i*)(wt + r * Cf::ROWB + (((s * 4 + gq) ^ r) << 4));
           const v8i wf = {w.x, w.y, w.z, w.w, 0, 0, 0, 0};
           const int wscale = (int)((uint32_t)sc[s / 4][s % 4] >> (8 * gq));
@@ -206,7 +205,6 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
     }
 
     // ---- reduce the 8 K-slices: partial sums meet in LDS (the ring is idle now) -----------------------
-    if constexpr ((VAR & 2) != 0) { if (acc[0][0].x == 1.2345f) ((float*)d.C)[0] = 1.f; continue; }
     __syncthreads();
     lds_v4f* const red = (lds_v4f*)smem;
 #pragma unroll
@@ -299,7 +297,7 @@ __device__ inline void issue_tile_dma2(const uint8_t* W, uint32_t wbytes, const 
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsS, (lds_void*)sdst, 16, soff, ssoff, 0, 0);
 }
 
-template <int XF, int SPW, typename OutT, int VAR = 0>
+template <int XF, int SPW, typename OutT>
 __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d) {
   using Cf = Decode2Cfg<SPW>;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
@@ -344,17 +342,12 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
     v4i xsraw[SPW / 4];
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
-      v4i lo, hi;
-      if constexpr ((VAR & 4) != 0) { lo = (v4i){s, 1, 2, 3}; hi = lo; }
-      else {
-        lo = __builtin_amdgcn_raw_buffer_load_b128(rsX, xoff, s * 128, 0);
-        hi = __builtin_amdgcn_raw_buffer_load_b128(rsX, xoff, s * 128 + 64, 0);
-      }
+      const v4i lo = __builtin_amdgcn_raw_buffer_load_b128(rsX, xoff, s * 128, 0);
+      const v4i hi = __builtin_amdgcn_raw_buffer_load_b128(rsX, xoff, s * 128 + 64, 0);
       xf[s] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     }
 #pragma unroll
     for (int u = 0; u < SPW / 4; ++u) {
-      if constexpr ((VAR & 4) != 0) { xsraw[u] = (v4i){u, 1, 2, 3}; continue; }
       xsraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rsXs, xsoff, u * 16, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -420,7 +413,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
     }
     __builtin_amdgcn_sched_barrier(0);
     // ... and so has everybody else's; the partial sums of tile i - 1 are all in LDS as well
-    if constexpr (!(VAR & 8)) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     // all of the tile's fragments and scales into registers, so that the slot can be refilled before the
     // multiplications start.  The scales first, packed to the lane's own byte of each K-step (one register
@@ -430,7 +423,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
     lds_u8* const st = smem + (i & 1) * Cf::SLOT + Cf::W_BYTES + r * Cf::SROW + q * (SPW * 4);
     int ws[SPW / 4];
     v4i w[SPW];
-    if constexpr (!(VAR & 1)) {
+    {
 #pragma unroll
       for (int h = 0; h < SPW / 4; ++h) {
         const v4i sc = *(lds_cv4i*)(st + 16 * h);
@@ -449,14 +442,13 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
       for (int s = 0; s < SPW; ++s) w[s] = *(lds_cv4i*)(wk[s & 3] + (s >> 2) * 256);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (!(VAR & 8)) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     if (i + 2 < t_count) issue(t_first + (i + 2) * G, i & 1);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (!(VAR & 2))
-      if (i > 0 && wave < 2) reduce_store(i - 1);   // uniform per wave
+    if (i > 0 && wave < 2) reduce_store(i - 1);   // uniform per wave
     v4f acc[2] = {(v4f){0.f, 0.f, 0.f, 0.f}, (v4f){0.f, 0.f, 0.f, 0.f}};   // even / odd K-steps: two MFMA chains
-    if constexpr (!(VAR & 1)) {
+    {
 #pragma unroll
       for (int s = 0; s < SPW; ++s) {
         const v8i wf = {w[s].x, w[s].y, w[s].z, w[s].w, 0, 0, 0, 0};
@@ -474,28 +466,13 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
     ((lds_v4f*)(smem + Cf::RING + (i & 1) * Cf::RED))[wave * 64 + lane] = acc[0] + acc[1];
   }
   __syncthreads();
-  if constexpr (!(VAR & 2))
-    if (wave < 2) reduce_store(t_count - 1);
+  if (wave < 2) reduce_store(t_count - 1);
 }
 
 template <int XF, int SPW, typename OutT>
 int launch_decode2_k(const DecodeArgs& d, int grid, hipStream_t stream) {
   using Cf = Decode2Cfg<SPW>;
   auto kern = decode2_kernel<XF, SPW, OutT>;
-#ifdef MXGEMM_TIMING_AIDS
-  // Only in builds made with -DMXGEMM_TIMING_AIDS: MXGEMM_DEC selects a variant with parts of the work removed
-  // (results invalid): 1 no MFMA / LDS reads, 2 no reduction, 4 no X loads, 8 no barriers
-  static const int var = [] { const char* e = getenv("MXGEMM_DEC"); return e ? atoi(e) : 0; }();
-  if constexpr (SPW == 16 && sizeof(OutT) == 2) {
-    if (var == 1) kern = decode2_kernel<XF, SPW, OutT, 1>;
-    if (var == 2) kern = decode2_kernel<XF, SPW, OutT, 2>;
-    if (var == 3) kern = decode2_kernel<XF, SPW, OutT, 3>;
-    if (var == 4) kern = decode2_kernel<XF, SPW, OutT, 4>;
-    if (var == 6) kern = decode2_kernel<XF, SPW, OutT, 6>;
-    if (var == 7) kern = decode2_kernel<XF, SPW, OutT, 7>;
-    if (var != 0) hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);
-  }
-#endif
   static int attr_done = 0;   // benign race: the attribute call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);
@@ -522,19 +499,6 @@ template <int XF, int SPW, int MT, typename OutT>
 int launch_decode_k(const DecodeArgs& d, int grid, hipStream_t stream) {
   using Cf = DecodeCfg<SPW, MT>;
   auto kern = decode_kernel<XF, SPW, MT, OutT>;
-#ifdef MXGEMM_TIMING_AIDS
-  // Only in builds made with -DMXGEMM_TIMING_AIDS (never the shipped library): MXGEMM_DEC selects a variant
-  // with parts of the work removed (results invalid): 1 no MFMA / LDS reads, 2 no reduction, 4 no X loads
-  static const int var = [] { const char* e = getenv("MXGEMM_DEC"); return e ? atoi(e) : 0; }();
-  if constexpr (SPW == 8 && MT == 2 && sizeof(OutT) == 2) {
-    if (var == 1) kern = decode_kernel<XF, SPW, MT, OutT, 1>;
-    if (var == 2) kern = decode_kernel<XF, SPW, MT, OutT, 2>;
-    if (var == 3) kern = decode_kernel<XF, SPW, MT, OutT, 3>;
-    if (var == 4) kern = decode_kernel<XF, SPW, MT, OutT, 4>;
-    if (var == 7) kern = decode_kernel<XF, SPW, MT, OutT, 7>;
-    if (var != 0) hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);
-  }
-#endif
   static int attr_done = 0;   // benign race: the attribute call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);
@@ -584,8 +548,7 @@ int launch_gemm_decode(const DecodeArgs& d, hipStream_t stream) {
   // the two-halves variant where its K-slices are whole (1024 or 2048 elements); with M <= 16 its second
   // half of the waves multiplies zeros but still carries half of the DMA, and it measures 1 - 4 % faster than
   // the 8-slice kernel there too (M = 1: 28.2 against 29.5 us on the 28672 x 8192 weights)
-  static const int two_env = [] { const char* e = getenv("MXGEMM_DECODE2"); return e ? atoi(e) : 1; }();
-  if (two_env && (d.K == 8192 || d.K == 4096))
+  if (d.K == 8192 || d.K == 4096)
     return d.x_fmt == MX_E4M3 ? launch_decode2_x<MX_E4M3>(d, grid, stream) : launch_decode2_x<MX_E5M2>(d, grid, stream);
   if (d.x_fmt == MX_E4M3) return launch_decode_x<MX_E4M3>(d, grid, stream);
   return launch_decode_x<MX_E5M2>(d, grid, stream);

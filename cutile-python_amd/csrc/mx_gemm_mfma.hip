@@ -32,7 +32,7 @@
 namespace mx {
 namespace {
 
-template <class C, typename OutT, bool GROUPED, int PIPE>
+template <class C, typename OutT, bool GROUPED>
 __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
   lds_u8* const smem = (lds_u8*)smem_generic;
@@ -92,7 +92,6 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
     const int col = (pos ^ swz<C::A_CPR>(row)) * 16;
     a_col[q] = col;
     int64_t grow = m0 + row;
-    if constexpr (PIPE == 6) grow = row & 15;          // timing experiment: every load hits in cache
     bool ok = grow < g.M;
     if constexpr (GROUPED) {
       const int id = ok ? g.sorted_token_ids[grow] : 0x7FFFFFFF;
@@ -108,7 +107,6 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
     const int col = (pos ^ swz<C::B_CPR>(row)) * 16;
     b_col[q] = col;
     int64_t grow = n0 + row;
-    if constexpr (PIPE == 6) grow = row & 15;
     b_voff[q] = grow < g.N ? (uint32_t)(grow * g.ldb + col) : kOobOffset;
   }
 
@@ -192,14 +190,9 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
       const int it = Qi * SPQ + t0 / C::KSUB;        // position in the (rotated) walk
       if (it < nstages) {
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this thread's LDS-DMA of stage s landed
-        if constexpr (PIPE != 4 && PIPE != 5)
-          __syncthreads();                    // everyone's landed; everyone left stage s-1's buffer
+        __syncthreads();                      // everyone's landed; everyone left stage s-1's buffer
         const bool more = it + 1 < nstages;
         const int sn = (t0 / C::KSUB + 1 < SPQ) ? s + 1 : Qn * SPQ;   // stage that follows in the walk
-        if constexpr (PIPE == 0) {
-#pragma unroll
-          for (int idx = 0; idx < TOTAL_LOADS; ++idx) issue_one(idx, sn, buf ^ 1, more);
-        }
         lds_u8* const atile = smem + buf * C::STAGE + (wm0 + r) * C::A_RB;
         lds_u8* const btile = smem + buf * C::STAGE + C::A_STAGE + (wn0 + r) * C::B_RB;
 #pragma unroll
@@ -207,14 +200,11 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
           v8i bf[C::NTL];
 #pragma unroll
           for (int j = 0; j < C::NTL; ++j) {
-            if constexpr (PIPE == 3 || PIPE == 5) bf[j] = (v8i){s, j, kk, gq, swb, lane, 3, 4};
-            else bf[j] = load_frag<C::B_RB, C::B_EB>(btile, 16 * j, kk, gq, swb);
+            bf[j] = load_frag<C::B_RB, C::B_EB>(btile, 16 * j, kk, gq, swb);
           }
 #pragma unroll
           for (int i = 0; i < C::MT; ++i) {
-            v8i af;
-            if constexpr (PIPE == 3 || PIPE == 5) af = (v8i){s, i, kk, gq, swa, lane, 1, 2};
-            else af = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
+            const v8i af = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
 #pragma unroll
             for (int j = 0; j < C::NTL; ++j) {
               // compile-time K-step index within the quad selects the scale byte
@@ -227,15 +217,13 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
               else
                 acc[i][j] = mfma_scaled<C::BF, C::AF, 3>(bf[j], af, acc[i][j], sb[j / 4][j % 4], sa[i / 4][i % 4]);
             }
-            if constexpr (PIPE == 1 || PIPE == 3 || PIPE == 6 || PIPE == 7) {
-              if (kk == 0 && i < LOAD_ITERS) {
+            if (kk == 0 && i < LOAD_ITERS) {
 #pragma unroll
-                for (int l = 0; l < LPI; ++l)
-                  if (i * LPI + l < (PIPE == 7 ? C::A_LOADS : TOTAL_LOADS)) issue_one(i * LPI + l, sn, buf ^ 1, more);
-              }
-              // keep the DMA loads in the tile iteration they were written in; everything else may move
-              __builtin_amdgcn_sched_barrier(0x78F);
+              for (int l = 0; l < LPI; ++l)
+                if (i * LPI + l < TOTAL_LOADS) issue_one(i * LPI + l, sn, buf ^ 1, more);
             }
+            // keep the DMA loads in the tile iteration they were written in; everything else may move
+            __builtin_amdgcn_sched_barrier(0x78F);
           }
         }
         buf ^= 1;
@@ -275,9 +263,9 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
   }
 }
 
-template <class C, typename OutT, bool GROUPED, int PIPE = 1>
+template <class C, typename OutT, bool GROUPED>
 int launch_one(const GemmArgs& g, hipStream_t stream) {
-  auto kern = gemm_kernel<C, OutT, GROUPED, PIPE>;
+  auto kern = gemm_kernel<C, OutT, GROUPED>;
   static int attr_done = 0;   // benign race: the attribute call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -300,26 +288,6 @@ template <int BM, int BN, int WGM, int WGN>
 int launch_fmt(const GemmArgs& g, hipStream_t stream) {
   const bool grouped = g.sorted_token_ids != nullptr;
   GemmArgs gs = g;
-#ifdef MXGEMM_TIMING_AIDS
-  // Only in builds made with -DMXGEMM_TIMING_AIDS (never the shipped library): MXGEMM_PIPE selects a variant
-  // with parts of the work removed (results invalid, except 0: all DMA loads of a stage in one burst);
-  // MXGEMM_STAGGER=1 starts every tile at a different K-quad
-  static const int pipe_env = [] { const char* e = getenv("MXGEMM_PIPE"); return e ? atoi(e) : 1; }();
-  static const int stagger_env = [] { const char* e = getenv("MXGEMM_STAGGER"); return e ? atoi(e) : 0; }();
-  gs.stagger = stagger_env;
-  if (pipe_env != 1 && g.a_fmt == MX_E4M3 && g.b_fmt == MX_E4M3 && g.c_dtype == MX_BF16 && !grouped) {
-    using C = Cfg<MX_E4M3, MX_E4M3, BM, BN, WGM, WGN>;
-    switch (pipe_env) {
-      case 0: return launch_one<C, uint16_t, false, 0>(gs, stream);
-      case 2: return launch_one<C, uint16_t, false, 2>(gs, stream);   // no DMA in the loop
-      case 3: return launch_one<C, uint16_t, false, 3>(gs, stream);   // no LDS reads
-      case 4: return launch_one<C, uint16_t, false, 4>(gs, stream);   // no DMA, no barrier
-      case 5: return launch_one<C, uint16_t, false, 5>(gs, stream);   // MFMA only
-      case 6: return launch_one<C, uint16_t, false, 6>(gs, stream);   // all loads cache-resident
-      case 7: return launch_one<C, uint16_t, false, 7>(gs, stream);   // only the A loads
-    }
-  }
-#endif
 #define MX_CASE(AFMT, BFMT)                                                                        \
   if (g.a_fmt == AFMT && g.b_fmt == BFMT) {                                                        \
     using C = Cfg<AFMT, BFMT, BM, BN, WGM, WGN>;                                                   \

@@ -95,7 +95,7 @@ struct TileWalk {
   }
 };
 
-template <class C, typename OutT, bool GROUPED, int TEAM, int VAR>
+template <class C, typename OutT, bool GROUPED, int TEAM>
 __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, const int wn,
                                         const int lane, const TileWalk& walk) {
   using P = PP<C>;
@@ -180,11 +180,8 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   // and the 16-byte chunks beyond the end of K read nothing and zero-fill their LDS bytes
   // (out-of-range buffer offset)
   auto issue_a = [&](int sl, int abuf) {
-    if constexpr (VAR & 1) return;
     lds_u8* const base = smem + abuf * C::A_STAGE + wm0 * C::A_RB + wn * 1024;
-    int sk = sl;
-    if constexpr (VAR & 8) sk &= 3;   // timing aid: every stage re-reads the first four (cache-resident)
-    const int ka = sk * C::A_RB;
+    const int ka = sl * C::A_RB;
     const int klim = sl < nstages ? Kb_a - ka : 0;   // bytes of this stage's rows that exist
 #pragma unroll
     for (int q = 0; q < AL; ++q) {
@@ -193,12 +190,9 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     }
   };
   auto issue_b = [&](int sl, int bbuf) {
-    if constexpr (VAR & 1) return;
     if constexpr (TEAM == 1) {
       lds_u8* const base = smem + P::B_BASE + bbuf * C::B_STAGE + wn0 * C::B_RB;
-      int sk = sl;
-      if constexpr (VAR & 8) sk &= 3;
-      const int kb = sk * C::B_RB;
+      const int kb = sl * C::B_RB;
       const int klim = sl < nstages ? Kb_b - kb : 0;
 #pragma unroll
       for (int q = 0; q < BL; ++q) {
@@ -227,7 +221,6 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   const bool accumulate = g.accumulate != 0;
   int eid[2] = {-1, -1};
   auto write_tile = [&](int m0, int n0) {
-    if constexpr ((VAR & 16) != 0) walk.origin(walk.first, m0, n0);   // timing aid: every tile to the same place
     if constexpr (!GROUPED) {
       // interior tile, plain store: one address per lane, everything else immediate offsets
       if (m0 + 256 <= g.M && n0 + 256 <= g.N && vec8_ok && !accumulate) {
@@ -236,7 +229,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
           for (int jp = 0; jp < 2; ++jp) {
-            if (!(VAR & 2) || g.ldc == -12345) store8_full<OutT>(p + 32 * jp, acc[i][2 * jp], acc[i][2 * jp + 1]);
+            store8_full<OutT>(p + 32 * jp, acc[i][2 * jp], acc[i][2 * jp + 1]);
             acc[i][2 * jp] = (v4f){0.f, 0.f, 0.f, 0.f};
             acc[i][2 * jp + 1] = (v4f){0.f, 0.f, 0.f, 0.f};
           }
@@ -252,8 +245,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
           t.v[i][j] = acc[i][j];
           acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
         }
-      if (!(VAR & 2) || g.ldc == -12345)
-        write_tile_checked<OutT>(t, Cp, g.ldc, g.M, g.N, m0 + wm0 + r, n0 + wn0 + 8 * gq, accumulate, vec_ok);
+      write_tile_checked<OutT>(t, Cp, g.ldc, g.M, g.N, m0 + wm0 + r, n0 + wn0 + 8 * gq, accumulate, vec_ok);
       return;
     }
     // grouped: row 16 i + c of the team's half goes to row `id` of C, where id is the routed-slot index
@@ -274,7 +266,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       if (g.topk_weights) w = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, ewt[i >> 2])));
       OutT* const p = Cp + (int64_t)id * g.ldc + (n0 + wn0 + 8 * gq);
       if (cols_in) {
-        if ((!(VAR & 2) || g.ldc == -12345) && ok) {
+        if (ok) {
 #pragma unroll
           for (int jp = 0; jp < 2; ++jp) store8_full<OutT>(p + 32 * jp, acc[i][2 * jp] * w, acc[i][2 * jp + 1] * w);
         }
@@ -282,7 +274,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int n = n0 + wn0 + 8 * gq + bperm_tile_off(j);
-          if ((!(VAR & 2) || g.ldc == -12345) && ok && n < g.N)
+          if (ok && n < g.N)
             store4<OutT>(p + bperm_tile_off(j), acc[i][j] * w, accumulate, g.N - n, vec_ok);
         }
       }
@@ -370,7 +362,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       // (the scale loads issued at the end of the previous quad are younger than those and may stay in
       // flight; the MFMA phase waits for them)
       constexpr int younger = (t0 == 0) ? P::SCALE_LOADS : 0;
-      if constexpr (!(VAR & 1)) __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL + BL + younger));
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL + BL + younger));
     }
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // fragments are in registers
@@ -382,8 +374,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       for (int kk = 0; kk < C::KSUB; ++kk)
 #pragma unroll
         for (int i = i0; i < i0 + 2; ++i) {
-          if constexpr (VAR & 4) af[kk][i] = af[kk][i & 1];
-          else af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
+          af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
         }
       __builtin_amdgcn_sched_barrier(0);
     };
@@ -425,7 +416,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (TEAM == 0 && !(VAR & 1)) {
+    if constexpr (TEAM == 0) {
       // A of stage s + 1 (issued one stage ago) must have landed; A of stage s + 2 and the scale
       // loads just issued may stay in flight
       __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL + (last_of_quad ? P::SCALE_LOADS : 0)));
@@ -457,7 +448,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   if constexpr (TEAM == 0) asm volatile("s_barrier" ::: "memory");   // pairs with team 1's extra barrier
 }
 
-template <class C, typename OutT, bool GROUPED, int VAR>
+template <class C, typename OutT, bool GROUPED>
 __global__ __launch_bounds__(512) void gemm_pp_kernel(const GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
   lds_u8* const smem = (lds_u8*)smem_generic;
@@ -481,9 +472,9 @@ __global__ __launch_bounds__(512) void gemm_pp_kernel(const GemmArgs g) {
   }
   if (walk.first >= walk.end) return;   // cannot happen with the grids the launcher picks
   if (wave < 4)
-    pp_body<C, OutT, GROUPED, 0, VAR>(g, smem, wave, lane, walk);
+    pp_body<C, OutT, GROUPED, 0>(g, smem, wave, lane, walk);
   else
-    pp_body<C, OutT, GROUPED, 1, VAR>(g, smem, wave - 4, lane, walk);
+    pp_body<C, OutT, GROUPED, 1>(g, smem, wave - 4, lane, walk);
 }
 
 int num_cus() {
@@ -496,9 +487,9 @@ int num_cus() {
   return cus;
 }
 
-template <class C, typename OutT, bool GROUPED, int VAR = 0>
+template <class C, typename OutT, bool GROUPED>
 int launch_pp(const GemmArgs& g, hipStream_t stream) {
-  auto kern = gemm_pp_kernel<C, OutT, GROUPED, VAR>;
+  auto kern = gemm_pp_kernel<C, OutT, GROUPED>;
   static int attr_done = 0;   // benign race: the attribute call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -515,9 +506,8 @@ int launch_pp(const GemmArgs& g, hipStream_t stream) {
   const int ksteps = (g.K + 127) / 128;
   const int nstages = (ksteps + C::KSUB - 1) / C::KSUB;
   const bool can_walk = nstages >= 2 && ksteps % 4 == 0;
-  static const int walk_env = [] { const char* e = getenv("MXGEMM_PP_WALK"); return e ? atoi(e) : 1; }();
   int64_t grid = tiles;
-  if (can_walk && walk_env && tiles > num_cus()) grid = num_cus();
+  if (can_walk && tiles > num_cus()) grid = num_cus();
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), PP<C>::LDS_BYTES, stream, g);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "gemm_pp_kernel launch: %s", hipGetErrorString(e));
@@ -530,38 +520,6 @@ int launch_gemm_pingpong(const GemmArgs& g, hipStream_t stream) {
   if (g.c_dtype != MX_F32 && g.c_dtype != MX_BF16)
     return set_error(MX_ERR_DTYPE, "MFMA kernel: output dtype %d not supported", g.c_dtype);
   const bool grouped = g.sorted_token_ids != nullptr;
-#ifdef MXGEMM_TIMING_AIDS
-  // Only in builds made with -DMXGEMM_TIMING_AIDS (never the shipped library): MXGEMM_PP_VAR, read once,
-  // selects a variant with parts of the work removed (results invalid): 1 no DMA in the loop, 2 no output
-  // stores, 4 no late LDS reads, 8 DMA of cache-resident data, 16 every tile of a workgroup stored to the
-  // place of its first one (cache-resident output)
-  static const int var_env = [] { const char* e = getenv("MXGEMM_PP_VAR"); return e ? (int)strtol(e, nullptr, 0) : 0; }();
-  if (var_env && g.a_fmt == MX_E4M3 && g.b_fmt == MX_E4M3 && g.c_dtype == MX_BF16) {
-    using C = Cfg<MX_E4M3, MX_E4M3, 256, 256, 2, 4>;
-    if (grouped) {
-      switch (var_env) {
-        case 1: return launch_pp<C, uint16_t, true, 1>(g, stream);
-        case 2: return launch_pp<C, uint16_t, true, 2>(g, stream);
-        case 4: return launch_pp<C, uint16_t, true, 4>(g, stream);
-        case 5: return launch_pp<C, uint16_t, true, 5>(g, stream);
-        case 7: return launch_pp<C, uint16_t, true, 7>(g, stream);
-        case 8: return launch_pp<C, uint16_t, true, 8>(g, stream);
-      }
-    } else {
-      switch (var_env) {
-        case 1: return launch_pp<C, uint16_t, false, 1>(g, stream);
-        case 2: return launch_pp<C, uint16_t, false, 2>(g, stream);
-        case 3: return launch_pp<C, uint16_t, false, 3>(g, stream);
-        case 4: return launch_pp<C, uint16_t, false, 4>(g, stream);
-        case 5: return launch_pp<C, uint16_t, false, 5>(g, stream);
-        case 7: return launch_pp<C, uint16_t, false, 7>(g, stream);
-        case 8: return launch_pp<C, uint16_t, false, 8>(g, stream);
-        case 10: return launch_pp<C, uint16_t, false, 10>(g, stream);
-        case 16: return launch_pp<C, uint16_t, false, 16>(g, stream);
-      }
-    }
-  }
-#endif
 #define MX_CASE(AFMT, BFMT)                                                                        \
   if (g.a_fmt == AFMT && g.b_fmt == BFMT) {                                                        \
     using C = Cfg<AFMT, BFMT, 256, 256, 2, 4>;                                                     \

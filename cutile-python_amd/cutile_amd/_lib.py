@@ -58,8 +58,13 @@ SYMBOLS = {
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32,
         ctypes.c_int64, _P(MxGemmOpts), ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
     "mx_moe_align_max_slots": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]),
+    "mx_moe_align_workspace_bytes": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int32]),
     "mx_moe_align": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32,
-                                    ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
+                                    ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                    ctypes.c_int64, ctypes.c_void_p]),
+    "mx_bench_gemm": (ctypes.c_int, [ctypes.c_int32] + [_P(MxTensor)] * 5 + [
+        _P(MxGemmOpts), ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32,
+        _P(ctypes.c_float), ctypes.c_void_p]),
     "mx_gemm_list_workspace_bytes": (ctypes.c_int64, [ctypes.c_int32, _P(MxTensor), _P(MxTensor), _P(MxGemmOpts)]),
     "mx_gemm_list": (ctypes.c_int, [ctypes.c_int32] + [_P(MxTensor)] * 5 + [_P(MxGemmOpts), ctypes.c_void_p,
                                     ctypes.c_int64, ctypes.c_void_p]),

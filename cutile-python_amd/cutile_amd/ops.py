@@ -18,6 +18,7 @@ Reference counterparts
 from __future__ import annotations
 
 import ctypes
+import threading
 from dataclasses import dataclass
 from typing import Optional, Tuple
 
@@ -144,25 +145,31 @@ def _scale_desc(s, rows: int, K: int, block: int, is_b: bool):
     return L.desc(_as_u8(s), code), L.MX_SCALE_2D
 
 
-_WS_CACHE: dict = {}
+_WS_LOCAL = threading.local()
 
 
 def _workspace(dev: torch.device, nbytes: int, stream: Optional[int] = None) -> Optional[torch.Tensor]:
-    """Scratch for the per-call scale re-layout: one buffer per (device, stream), grown on demand, so the
-    hot path does not go through the allocator.  Kernels that use it are ordered on that stream."""
+    """Scratch for the per-call scale re-layout: one buffer per (host thread, device, stream), grown on
+    demand, so the hot path does not go through the allocator.  The kernels that use a buffer are ordered
+    on its stream, and no other host thread is ever handed the same buffer, so concurrent callers cannot
+    overwrite each other's scales between the re-layout launch and the GEMM launch.  While the stream is
+    being captured into a graph the buffer comes fresh from the allocator (the capture's private pool) and
+    is not cached: a cached one would later be reused by eager calls while replays of the graph still
+    write to it."""
     if nbytes <= 0:
         return None
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    cache = _WS_LOCAL.__dict__.setdefault("buffers", {})
     key = (dev.index, L.stream_ptr(dev) if stream is None else stream)
-    buf = _WS_CACHE.get(key)
+    buf = cache.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
-        _WS_CACHE[key] = buf
+        cache[key] = buf
     return buf
 
 
-def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kernel, block, split_k=0):
-    dev = A.device
-    and_, bnd = A.dim(), B.dim()
+def _gemm_descs(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, block):
     a_log = _logical_shape(A, a_pd if a_fmt == "e2m1" else -1)
     b_log = _logical_shape(B, b_pd if b_fmt == "e2m1" else -1)
     M, K, N = a_log[-2], a_log[-1], b_log[-1]
@@ -171,6 +178,12 @@ def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kerne
     dAs, la = _scale_desc(As, M, K, block, False)
     dBs, lb = _scale_desc(Bs, N, K, block, True)
     dC = L.desc(C, L._TORCH_TO_MX[C.dtype])
+    return (dA, dAs, dB, dBs, dC), (la, lb), (M, N, K)
+
+
+def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kernel, block, split_k=0):
+    dev = A.device
+    (dA, dAs, dB, dBs, dC), (la, lb), (M, N, K) = _gemm_descs(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, block)
     o = _opts(accumulate, la, lb, kernel, block, split_k)
     lib = L.lib()
     need = lib.mx_gemm_workspace_bytes(M, N, K, ctypes.byref(o))
@@ -185,6 +198,49 @@ def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kerne
             rc = lib.mx_gemm(*args)
     _check(rc)
     return C
+
+
+def bench_block_scaled_matmul(operand_sets, *, warmup: int = 5, iters: int = 20, kernel: str = "auto",
+                              a_format: Optional[str] = None, b_format: Optional[str] = None):
+    """Times ``block_scaled_matmul(A, A_scale, B, B_scale, C=C)`` the way the reference's tuner times a kernel
+    (``_benchmark``, cext/tile_kernel.cpp:3921-4042; protocol of src/cuda/tile/tune/_tune.py:339-395): every
+    call between its own pair of HIP events on the current stream.  ``operand_sets`` is a list of
+    ``(A, A_scale, B, B_scale, C)`` tuples of one problem shape; call i uses set i % len(operand_sets), which
+    takes the place of the reference's cache-flushing memset.  Returns the ``iters`` durations in
+    milliseconds (a list of floats); synchronises the stream."""
+    n = len(operand_sets)
+    if n == 0:
+        raise TileValueError("bench_block_scaled_matmul needs at least one operand set")
+    arr = [(L.MxTensor * n)() for _ in range(5)]
+    layouts, dims, keep = set(), set(), []
+    dev = operand_sets[0][0].device
+    for i, (A, As, B, Bs, C) in enumerate(operand_sets):
+        a_fmt, b_fmt = _elem_format(A, a_format), _elem_format(B, b_format)
+        if a_fmt is None or b_fmt is None:
+            raise TileTypeError("Unsupported input dtype for mma_scaled, supported input dtypes are "
+                                "float8_e4m3fn, float8_e5m2, float4_e2m1fn")
+        a_pd = _packed_dim(A, 1, None) if a_fmt == "e2m1" else -1
+        b_pd = _packed_dim(B, 0, None) if b_fmt == "e2m1" else -1
+        descs, lay, mnk = _gemm_descs(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, 32)
+        for j in range(5):
+            arr[j][i] = descs[j]
+        layouts.add(lay)
+        dims.add(mnk)
+        keep.append((A, As, B, Bs, C))
+    if len(layouts) != 1 or len(dims) != 1:
+        raise TileValueError("all operand sets must share one problem shape and one scale layout")
+    (la, lb), (M, N, K) = layouts.pop(), dims.pop()
+    o = _opts(False, la, lb, kernel, 32)
+    lib = L.lib()
+    need = lib.mx_gemm_workspace_bytes(M, N, K, ctypes.byref(o))
+    stream = L.stream_ptr(dev)
+    ws = _workspace(dev, need, stream)
+    times = (ctypes.c_float * iters)()
+    with torch.cuda.device(dev):
+        rc = lib.mx_bench_gemm(n, arr[0], arr[1], arr[2], arr[3], arr[4], ctypes.byref(o),
+                               ws.data_ptr() if ws is not None else None, need, warmup, iters, times, stream)
+    _check(rc)
+    return list(times)
 
 
 # ==================================================================================================
@@ -515,9 +571,12 @@ def moe_align_tile_size(topk_ids: torch.Tensor, tile_m: int, num_experts: int, *
     ids = torch.empty(max_slots, dtype=torch.int32, device=flat.device)
     eids = torch.empty(max_slots // tile_m, dtype=torch.int32, device=flat.device)
     used = torch.zeros(1, dtype=torch.int32, device=flat.device)
+    need = lib.mx_moe_align_workspace_bytes(n, num_experts)
+    ws = _workspace(flat.device, need)
     with torch.cuda.device(flat.device):
         rc = lib.mx_moe_align(flat.data_ptr(), n, num_experts, tile_m, ids.data_ptr(), eids.data_ptr(),
-                              used.data_ptr(), L.stream_ptr(flat.device))
+                              used.data_ptr(), ws.data_ptr() if ws is not None else None, need,
+                              L.stream_ptr(flat.device))
     _check(rc)
     if exact:
         u = int(used.item())

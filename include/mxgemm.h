@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define MXGEMM_VERSION 100
+#define MXGEMM_VERSION 101
 
 /* Exported symbols (the library is built with hidden default visibility). */
 #if defined(__GNUC__)
@@ -138,8 +138,8 @@ MX_API int64_t mx_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, const mx
  *   C  [M,N]  MX_F32 | MX_BF16
  * The MFMA kernels need K-contiguous A (stride[1]==1) and B (stride[0]==1), 16-byte aligned rows
  * and block_size 32; MX_KERNEL_AUTO falls back to the generic kernel otherwise.
- * Optional leading batch dimension (ndim 3) is handled by the generic kernel with broadcast of
- * size-1 batches (test/test_mma_scaled.py:128-145).
+ * Optional leading batch dimension (ndim 3, test/test_mma_scaled.py:128-145): one 2-D product per batch
+ * entry on the same kernels, batches of size 1 broadcast; the entries share the workspace in stream order.
  */
 MX_API int mx_gemm(const mx_tensor* A, const mx_tensor* A_scale, const mx_tensor* B,
             const mx_tensor* B_scale, mx_tensor* C, const mx_gemm_opts* opts, void* workspace,
@@ -159,6 +159,20 @@ MX_API int64_t mx_gemm_list_workspace_bytes(int32_t count, const mx_tensor* A, c
 MX_API int mx_gemm_list(int32_t count, const mx_tensor* A, const mx_tensor* A_scale, const mx_tensor* B,
                  const mx_tensor* B_scale, mx_tensor* C, const mx_gemm_opts* opts, void* workspace,
                  int64_t workspace_bytes, void* stream);
+
+/*
+ * Timing aid, the counterpart of the reference launcher's _benchmark (cext/tile_kernel.cpp:3921-4042, used by
+ * the tuner, src/cuda/tile/tune/_tune.py:339-395): `warmup` untimed mx_gemm calls, then `iters` calls, each
+ * between its own pair of HIP events recorded on `stream`; times_ms[i] (host memory, `iters` floats) receives the
+ * duration of call i, which includes whatever mx_gemm enqueues for it (scale re-layout unless the scales are
+ * MX_SCALE_NATIVE).  Where the reference defeats the cache by writing an L2-sized buffer before each timed
+ * launch, this rotates operand sets: the descriptor arrays hold `nsets` entries each and call i uses set
+ * i % nsets, so give it enough distinct sets to exceed the 256 MiB Infinity Cache.  The only entry point that
+ * synchronises: it returns after `stream` has drained.  Creates HIP events; allocates no device memory.
+ */
+MX_API int mx_bench_gemm(int32_t nsets, const mx_tensor* A, const mx_tensor* A_scale, const mx_tensor* B,
+                  const mx_tensor* B_scale, mx_tensor* C, const mx_gemm_opts* opts, void* workspace,
+                  int64_t workspace_bytes, int32_t warmup, int32_t iters, float* times_ms, void* stream);
 
 /*
  * Grouped (MoE) variant.  Replaces: ct.launch(..., fused_moe_kernel, (A, B, C, topk_weights,
@@ -187,12 +201,16 @@ MX_API int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* A_scale, const m
  * sentinel value num_ids.  Outputs must hold mx_moe_align_max_slots(num_ids, num_experts, tile_m)
  * int32 slots and that number / tile_m blocks; unused trailing slots are filled with the sentinel
  * and unused trailing blocks with expert 0.  *num_slots_out (device int32, optional) receives the
- * number of slots actually used.  No host synchronisation.
+ * number of slots actually used.  No host synchronisation, no atomics on global memory, every output
+ * element written exactly once.
  */
 MX_API int64_t mx_moe_align_max_slots(int64_t num_ids, int32_t num_experts, int32_t tile_m);
+/* Scratch for the per-chunk histograms of mx_moe_align: 0 for up to 1024 ids (one workgroup), otherwise
+ * chunks x num_experts int32 (the ids are sorted by up to 256 workgroups, more beyond 16.7 M ids). */
+MX_API int64_t mx_moe_align_workspace_bytes(int64_t num_ids, int32_t num_experts);
 MX_API int mx_moe_align(const int32_t* topk_ids, int64_t num_ids, int32_t num_experts, int32_t tile_m,
                  int32_t* sorted_token_ids, int32_t* sorted_expert_ids, int32_t* num_slots_out,
-                 void* stream);
+                 void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
  * MX quantisation of the last axis in blocks of 32 (replaces the torch-op sequence of

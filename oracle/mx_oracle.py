@@ -210,7 +210,9 @@ def block_quantize(x: np.ndarray, block_size: int = 32, fmt: str = E4M3, scale_m
     xb = _blocks(x, block_size)
     amax = np.max(np.abs(xb), axis=-1, keepdims=True).astype(np.float32)
     if scale_mode == "ceil":
-        v = np.maximum((amax / np.float32(448.0)).astype(np.float32), np.float32(1e-12))
+        with np.errstate(invalid="ignore"):
+            v = np.maximum((amax / np.float32(448.0)).astype(np.float32), np.float32(1e-12))
+        v = np.where(np.isfinite(v), v, np.float32(1.0))   # non-finite blocks are overwritten below
         m, e = np.frexp(v)                       # v = m * 2^e, m in [0.5, 1)
         se = np.where(m == 0.5, e - 1, e).astype(np.int32)   # exact ceil(log2 v)
         saturate = False
@@ -232,8 +234,26 @@ def block_quantize(x: np.ndarray, block_size: int = 32, fmt: str = E4M3, scale_m
         codes = encode_e2m1(q)
     else:
         raise ValueError(fmt)
+    scale_bytes = (se[..., 0] + 127).astype(np.uint8)
+    if scale_mode == "ceil" and not np.all(np.isfinite(amax)):
+        # Non-finite blocks under the reference's rule (kernel_utils.py:69-78 evaluated by torch): clamp(min=)
+        # keeps NaN and inf / 448 is inf, so the scale is NaN or inf and its float8_e8m0fnu byte is 0xFF;
+        # x / scale is NaN for every element of a NaN block (an element that is NaN itself keeps its sign),
+        # and in an inf block NaN with the sign bit set where |x| is inf (inf / inf) and a signed zero
+        # elsewhere.  E2M1 has no NaN: non-finite elements saturate to +-6.
+        nf = ~np.isfinite(amax)
+        blk_nan = np.isnan(amax)
+        a_nan, a_inf = np.isnan(xb), np.isinf(xb)
+        sgn = np.signbit(xb).astype(np.uint8)
+        if fmt == E2M1:
+            special = (sgn << 3) | np.where(blk_nan | a_inf, np.uint8(7), np.uint8(0))
+        else:
+            special = np.where(a_nan, (sgn << 7) | np.uint8(0x7F),
+                               np.where(blk_nan, np.uint8(0x7F), np.where(a_inf, np.uint8(0xFF), sgn << 7)))
+        codes = np.where(nf, special.astype(np.uint8), codes.reshape(xb.shape))
+        scale_bytes = np.where(nf[..., 0], np.uint8(0xFF), scale_bytes)
     codes = codes.reshape(*xb.shape[:-2], xb.shape[-2] * block_size)
-    return codes, (se[..., 0] + 127).astype(np.uint8)
+    return codes, scale_bytes.astype(np.uint8)
 
 
 # ----------------------------------------------------------------------------------------------

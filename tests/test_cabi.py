@@ -84,6 +84,20 @@ def test_validation_codes_without_gpu():
     rc = lib.mx_gemm(ctypes.byref(A), ctypes.byref(As), ctypes.byref(Brm), ctypes.byref(Bs), ctypes.byref(C),
                      ctypes.byref(o), None, 0, None)
     assert rc == L.MX_ERR_LAYOUT and "K axis is not contiguous" in L.last_error()
+    # the general kernel validates a swizzle_32_4_4 descriptor before it indexes through it
+    o = L.MxGemmOpts(struct_size=32, kernel=L.MX_KERNEL_GENERIC, block_size=32,
+                     a_scale_layout=L.MX_SCALE_SWIZZLE_32_4_4)
+    A128 = _desc(p, L.MX_E4M3, (128, 128), (128, 1))
+    C128 = _desc(p, L.MX_F32, (128, 32), (32, 1))
+    for bad in (_desc(p, L.MX_E8M0, (128, 4), (4, 1)), _desc(p, L.MX_E8M0, (2, 1, 32, 16), (512, 512, 16, 1)),
+                _desc(p, L.MX_E8M0, (1, 1, 32, 16), (512, 512, 32, 2))):
+        rc = lib.mx_gemm(ctypes.byref(A128), ctypes.byref(bad), ctypes.byref(B), ctypes.byref(Bs), ctypes.byref(C128),
+                         ctypes.byref(o), None, 0, None)
+        assert rc in (L.MX_ERR_SHAPE, L.MX_ERR_LAYOUT), (rc, L.last_error())
+    # moe_align: scratch for more than one chunk of ids is required
+    assert lib.mx_moe_align_workspace_bytes(1024, 8) == 0
+    assert lib.mx_moe_align_workspace_bytes(8192, 8) == 8 * 8 * 4
+    assert lib.mx_moe_align(p, 8192, 8, 256, p, p, None, None, 0, None) == L.MX_ERR_WORKSPACE
     # quantiser argument checks
     x = _desc(p, L.MX_F32, (4, 16), (16, 1))
     xq = _desc(p, L.MX_E4M3, (4, 32), (32, 1))

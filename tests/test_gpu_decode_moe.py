@@ -60,6 +60,27 @@ def test_moe_align_matches_oracle(ct, dev, T, topk, E, tile):
     assert bool((all_ids[len(want_ids):] == T * topk).all()) and bool((all_e[len(want_e):] == 0).all())
 
 
+@pytest.mark.parametrize("n,E,tile,skew", [(200_000, 3, 256, True), (70_000, 1, 128, False), (300_000, 300, 64, True),
+                                          (5000, 8, 256, False), (1025, 5, 16, False), (1024, 5, 16, False)])
+def test_moe_align_many_ids_per_expert(ct, dev, n, E, tile, skew):
+    """Routings that span many workgroups: one expert holding more than 65535 ids (a 16-bit running count
+    would wrap), more than 256 experts (the ballot placement) over several chunks, and sizes either side of
+    the one-workgroup limit."""
+    rng = np.random.default_rng(n + E)
+    if skew:
+        p = np.full(E, 0.1 / max(E - 1, 1))
+        p[E // 2] = 0.9
+        ids = rng.choice(E, size=n, p=p / p.sum()).astype(np.int32)
+    else:
+        ids = rng.integers(0, E, size=n, dtype=np.int32)
+    want_ids, want_e = O.moe_align_tile_size(ids.reshape(-1, 1), tile, E)
+    got_ids, got_e = ct.moe_align_tile_size(torch.from_numpy(ids).to(dev).reshape(-1, 1), tile, E)
+    assert np.array_equal(got_ids.cpu().numpy(), want_ids)
+    assert np.array_equal(got_e.cpu().numpy(), want_e)
+    all_ids, all_e = ct.moe_align_tile_size(torch.from_numpy(ids).to(dev).reshape(-1, 1), tile, E, exact=False)
+    assert bool((all_ids[len(want_ids):] == n).all()) and bool((all_e[len(want_e):] == 0).all())
+
+
 def _moe_case(T, K, N, E, topk, seed, dev, w_std=0.1):
     a = randn_operand(T, K, O.E4M3, seed, dev, std=0.5)
     w = randn_operand(E * N, K, O.E4M3, seed + 1, dev, std=w_std)

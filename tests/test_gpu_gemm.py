@@ -132,27 +132,53 @@ def test_auto_dispatch_matches_explicit(ct, dev):
 
 
 def test_concurrent_launch_threads(ct, dev):
-    """test/test_concurrent_launch.py:49-72: several Python threads launching at once."""
+    """test/test_concurrent_launch.py:49-72: several Python threads launching at once.  Every thread has its
+    own operands and scales (different shapes too), so a scale re-layout of one thread landing between
+    another thread's re-layout and GEMM launches would show as a wrong result."""
     import threading
-    a = randn_operand(128, 256, O.E4M3, 71, dev)
-    b = randn_operand(128, 256, O.E4M3, 72, dev)
-    want = _run(ct, a, b)
+    cases = []
+    for t in range(8):
+        a = randn_operand(128 + 64 * (t % 3), 256 + 128 * (t % 2), O.E4M3, 710 + t, dev, std=1.0 + t)
+        b = randn_operand(128 + 32 * (t % 4), 256 + 128 * (t % 2), O.E4M3, 720 + t, dev)
+        cases.append((a, b, _run(ct, a, b)))
+    torch.cuda.synchronize()
     errs = []
 
-    def work():
+    def work(t):
+        a, b, want = cases[t]
         try:
-            for _ in range(50):
-                c = _run(ct, a, b)
+            outs = [_run(ct, a, b) for _ in range(50)]
             torch.cuda.synchronize()
-            if not torch.equal(c, want):
-                errs.append("mismatch")
+            if not all(torch.equal(c, want) for c in outs):
+                errs.append(f"thread {t}: mismatch")
         except Exception as e:  # noqa: BLE001
             errs.append(repr(e))
 
-    ts = [threading.Thread(target=work) for _ in range(8)]
+    ts = [threading.Thread(target=work, args=(t,)) for t in range(8)]
     [t.start() for t in ts]
     [t.join() for t in ts]
     assert not errs, errs
+    for a, b, want in cases:
+        _check(want, oracle_matmul(a, b), torch.float32, "threads")
+
+
+@pytest.mark.parametrize("kernel", ["generic"] + MFMA + ["auto"])
+def test_config_c1_mxfp8_512_floor_fp32(ct, dev, kernel):
+    """The CPU-reference configuration of the metric: M = N = K = 512, A and B^T drawn N(0, 1) from seed 1234,
+    quantised by the oracle with the floor rule, fp32 output, every kernel; the input recipe and the check
+    mirror samples/BlockScaledMatMul.py:323-364."""
+    g = torch.Generator().manual_seed(1234)
+    a = torch.randn((512, 512), generator=g)
+    bt = torch.randn((512, 512), generator=g)
+    ac, asc = O.block_quantize(a.numpy(), 32, O.E4M3, "floor")
+    bc, bsc = O.block_quantize(bt.numpy(), 32, O.E4M3, "floor")
+    A, B = Operand(ac, asc, O.E4M3, dev), Operand(bc, bsc, O.E4M3, dev)
+    ref = oracle_matmul(A, B)
+    c = _run(ct, A, B, out_dtype=torch.float32, kernel=kernel)
+    _check(c, ref, torch.float32, f"C1 {kernel}")
+    # the device quantiser produces the same operands from the same fp32 inputs
+    aq, asq = ct.block_quantize(a.to(dev), 32, scale_mode="floor")
+    assert np.array_equal(aq.view(torch.uint8).cpu().numpy(), ac) and np.array_equal(asq.view(torch.uint8).cpu().numpy(), asc)
 
 
 @pytest.mark.parametrize("kernel", ["auto", "generic", "mfma128"])

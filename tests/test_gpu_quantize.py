@@ -81,7 +81,7 @@ def test_quantize_dequantize_roundtrip_large(ct, dev):
     assert torch.equal(xq2.view(torch.uint8), q)
 
 
-def _native_layout(scales: np.ndarray) -> np.ndarray:
+def _native_layout_loops(scales: np.ndarray) -> np.ndarray:
     """Plain-numpy statement of the native scale layout: dword [I/4][Q][lane][I%4], byte t = scale of row
     16 I + lane%16, block (4Q + t)*4 + lane/16; padding byte 127."""
     R, KB = scales.shape
@@ -96,13 +96,15 @@ def _native_layout(scales: np.ndarray) -> np.ndarray:
     return out.reshape(-1)
 
 
-@pytest.mark.parametrize("R,K", [(64, 512), (100, 160), (256, 1024), (16, 32)])
-def test_pack_scales_layout(ct, dev, R, K):
+@pytest.mark.parametrize("R,K", [(64, 512), (100, 160), (256, 1024), (16, 32), (128, 128), (384, 2048)])
+def test_pack_scales_layout_all_sources_agree(ct, dev, R, K):
+    """Element-by-element statement of the layout, and the same bytes from every source form: row-major,
+    transposed (how B_scale is passed) and the 4-D swizzle_32_4_4 tensor."""
     rng = np.random.default_rng(R + K)
     s = rng.integers(0, 255, (R, K // 32), dtype=np.uint8)
     t = torch.from_numpy(s).to(dev)
     p = ct.pack_scales(t.view(torch.float8_e8m0fnu))
-    want = _native_layout(s)
+    want = _native_layout_loops(s)
     got = p.data.cpu().numpy()[:want.size]
     assert np.array_equal(got, want)
     # transposed source (how B_scale is passed) gives the same bytes
@@ -208,3 +210,27 @@ def test_quantize_dense_rounding_grid(ct, dev, fmt, mode):
         got_codes = O.unpack_fp4(got_codes)
     assert np.array_equal(got_s.view(torch.uint8).cpu().numpy(), want_s)
     assert np.array_equal(got_codes, want_q)
+
+
+@pytest.mark.parametrize("dt", [torch.float8_e4m3fn, torch.float8_e5m2], ids=str)
+def test_quantize_nonfinite_blocks_follow_the_reference_rule(ct, dev, dt):
+    """Blocks holding NaN or inf under the reference's rule (test/kernels/kernel_utils.py:69-78 as torch
+    evaluates it): scale byte 0xFF, NaN codes where x / scale is NaN, signed zeros elsewhere.  Compared with
+    the literal torch restatement on the CPU, and with the oracle's integer formulation."""
+    x = np.random.default_rng(0).standard_normal((8, 96)).astype(np.float32)
+    x[0, 3] = np.nan
+    x[1, 5] = np.inf
+    x[2, 40] = -np.inf
+    x[3, 1] = -np.float32(np.nan)
+    x[3, 2] = np.inf
+    x[4, 33] = np.inf
+    x[4, 34] = -np.inf
+    x[5, 64:96] = np.nan
+    lit_q, lit_s = O.block_quantize_ceil_literal(torch.from_numpy(x), 32, dt)
+    got_q, got_s = ct.block_quantize(torch.from_numpy(x).to(dev), 32, dt, scale_mode="ceil")
+    assert np.array_equal(got_s.view(torch.uint8).cpu().numpy(), lit_s.view(torch.uint8).numpy())
+    assert np.array_equal(got_q.view(torch.uint8).cpu().numpy(), lit_q.view(torch.uint8).numpy())
+    fmt = O.E4M3 if dt == torch.float8_e4m3fn else O.E5M2
+    codes, sb = O.block_quantize(x, 32, fmt, "ceil")
+    assert np.array_equal(got_s.view(torch.uint8).cpu().numpy(), sb)
+    assert np.array_equal(got_q.view(torch.uint8).cpu().numpy(), codes)
