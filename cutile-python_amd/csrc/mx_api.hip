@@ -4,7 +4,14 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "mx_common.h"
+
+// Scratch of mx_gemm_static: lives in the library's device image, one copy per GPU the library runs on, held
+// until the process ends.  Host code never uses this name as an address: static_scratch() below resolves the
+// device address once per device with hipGetSymbolAddress and everything else uses that pointer.
+static __device__ __align__(256) unsigned char scratch[MX_STATIC_SCRATCH_BYTES];
 
 namespace mx {
 
@@ -88,6 +95,25 @@ const char* mfma_operand_issue(const void* ptr, int64_t rows, int64_t ld_bytes, 
   return nullptr;
 }
 
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// device address of `scratch` on the current device (each GPU holds its own copy at its own address)
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return set_error(MX_ERR_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return set_error(MX_ERR_DEVICE, "device index %d out of range", dev);
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return set_error(MX_ERR_DEVICE, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev].store(p, std::memory_order_release);   // a racing thread stores the same address
+  }
+  *out = p;
+  return MX_OK;
+}
 }  // namespace
 }  // namespace mx
 
@@ -108,7 +134,8 @@ int mx_device_check(void) {
   if (e != hipSuccess) return set_error(MX_ERR_DEVICE, "hipGetDeviceProperties: %s", hipGetErrorString(e));
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return set_error(MX_ERR_DEVICE, "libmxgemm is built for gfx950 only, device is %s", prop.gcnArchName);
-  return MX_OK;
+  void* p = nullptr;
+  return static_scratch(&p);   // set-up of mx_gemm_static on this device
 }
 
 int64_t mx_packed_scale_bytes(int64_t rows, int64_t K) {
@@ -455,6 +482,25 @@ void problem_dims(const mx_tensor& A, const mx_tensor& B, int64_t& M, int64_t& N
   N = bn >= 2 ? B.shape[bn - 1] : 0;
 }
 }  // namespace
+
+int64_t mx_static_scratch_bytes(void) { return MX_STATIC_SCRATCH_BYTES; }
+
+int mx_gemm_static(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const mx_tensor* Bs, mx_tensor* C,
+                   const mx_gemm_opts* opts, void* stream) {
+  if (!A || !B) return set_error(MX_ERR_INVALID, "mx_gemm_static: null descriptor");
+  if (A->ndim < 2 || A->ndim > 3 || B->ndim < 2 || B->ndim > 3)
+    return set_error(MX_ERR_SHAPE, "mx_gemm_static: A and B must have 2 or 3 dimensions");
+  int64_t M, N, K;
+  problem_dims(*A, *B, M, N, K);
+  const int64_t need = mx_gemm_workspace_bytes(M, N, K, opts);
+  if (need > MX_STATIC_SCRATCH_BYTES)
+    return set_error(MX_ERR_WORKSPACE, "mx_gemm_static: this problem needs %lld bytes of scratch, the static buffer "
+                     "holds %lld; use mx_gemm with a caller-owned workspace", (long long)need,
+                     (long long)MX_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  return mx_gemm(A, As, B, Bs, C, opts, ws, MX_STATIC_SCRATCH_BYTES, stream);
+}
 
 int64_t mx_gemm_list_workspace_bytes(int32_t count, const mx_tensor* A, const mx_tensor* B,
                                      const mx_gemm_opts* opts) {

@@ -53,6 +53,8 @@ SYMBOLS = {
     "mx_gemm_workspace_bytes": (ctypes.c_int64, [ctypes.c_int64] * 3 + [_P(MxGemmOpts)]),
     "mx_gemm": (ctypes.c_int, [_P(MxTensor)] * 5 + [_P(MxGemmOpts), ctypes.c_void_p, ctypes.c_int64,
                                                    ctypes.c_void_p]),
+    "mx_static_scratch_bytes": (ctypes.c_int64, []),
+    "mx_gemm_static": (ctypes.c_int, [_P(MxTensor)] * 5 + [_P(MxGemmOpts), ctypes.c_void_p]),
     "mx_gemm_grouped_workspace_bytes": (ctypes.c_int64, [ctypes.c_int64] * 4 + [_P(MxGemmOpts)]),
     "mx_gemm_grouped": (ctypes.c_int, [_P(MxTensor)] * 5 + [
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32,

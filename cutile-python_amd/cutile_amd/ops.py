@@ -181,21 +181,30 @@ def _gemm_descs(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, block):
     return (dA, dAs, dB, dBs, dC), (la, lb), (M, N, K)
 
 
-def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kernel, block, split_k=0):
+def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kernel, block, split_k=0,
+                 static_scratch=False):
     dev = A.device
     (dA, dAs, dB, dBs, dC), (la, lb), (M, N, K) = _gemm_descs(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, block)
     o = _opts(accumulate, la, lb, kernel, block, split_k)
     lib = L.lib()
-    need = lib.mx_gemm_workspace_bytes(M, N, K, ctypes.byref(o))
     stream = L.stream_ptr(dev)
-    ws = _workspace(dev, need, stream)
-    args = (ctypes.byref(dA), ctypes.byref(dAs), ctypes.byref(dB), ctypes.byref(dBs), ctypes.byref(dC),
-            ctypes.byref(o), ws.data_ptr() if ws is not None else None, need, stream)
+    if static_scratch:
+        fn = lib.mx_gemm_static
+        args = (ctypes.byref(dA), ctypes.byref(dAs), ctypes.byref(dB), ctypes.byref(dBs), ctypes.byref(dC),
+                ctypes.byref(o), stream)
+    else:
+        fn = lib.mx_gemm
+        need = lib.mx_gemm_workspace_bytes(M, N, K, ctypes.byref(o))
+        ws = _workspace(dev, need, stream)
+        args = (ctypes.byref(dA), ctypes.byref(dAs), ctypes.byref(dB), ctypes.byref(dBs), ctypes.byref(dC),
+                ctypes.byref(o), ws.data_ptr() if ws is not None else None, need, stream)
     if torch.cuda.current_device() == dev.index:
-        rc = lib.mx_gemm(*args)
+        rc = fn(*args)
     else:
         with torch.cuda.device(dev):
-            rc = lib.mx_gemm(*args)
+            rc = fn(*args)
+    if rc == L.MX_ERR_WORKSPACE:
+        raise ValueError(L.last_error())
     _check(rc)
     return C
 
@@ -249,7 +258,8 @@ def bench_block_scaled_matmul(operand_sets, *, warmup: int = 5, iters: int = 20,
 def block_scaled_matmul(A: torch.Tensor, A_scale, B: torch.Tensor, B_scale, *,
                         out_dtype: torch.dtype = torch.float32, C: Optional[torch.Tensor] = None,
                         accumulate: bool = False, a_format: Optional[str] = None,
-                        b_format: Optional[str] = None, kernel: str = "auto", split_k: int = 0) -> torch.Tensor:
+                        b_format: Optional[str] = None, kernel: str = "auto", split_k: int = 0,
+                        static_scratch: bool = False) -> torch.Tensor:
     """C = (A * A_scale) @ (B * B_scale) with fp32 accumulation, returned as ``out_dtype``.
 
     A (M, K) and B (K, N) hold MX elements: ``float8_e4m3fn`` / ``float8_e5m2``, or FP4 E2M1 packed two
@@ -261,6 +271,10 @@ def block_scaled_matmul(A: torch.Tensor, A_scale, B: torch.Tensor, B_scale, *,
     K-contiguous operands, i.e. B given as the transposed view of an (N, K) tensor as the reference
     sample does; other layouts run on a slower general kernel.  ``split_k``: 0 lets the library split a
     long K over several workgroups when M x N alone cannot fill the GPU, 1 forbids it, n > 1 forces n slices.
+    ``static_scratch``: take the scratch for the scale re-layout from the library's fixed per-GPU buffer
+    (``mx_gemm_static``) instead of a torch allocation; with a preallocated ``C`` the call then allocates
+    nothing.  Problems that need more than ``lib().mx_static_scratch_bytes()`` raise ``ValueError``; calls that
+    overlap on one GPU (several streams or threads) must not share it.
     """
     a_fmt, b_fmt = _elem_format(A, a_format), _elem_format(B, b_format)
     if a_fmt is None or b_fmt is None:
@@ -297,7 +311,7 @@ def block_scaled_matmul(A: torch.Tensor, A_scale, B: torch.Tensor, B_scale, *,
         if tuple(C.shape) != (m, n) or C.dtype not in (torch.float32, torch.bfloat16) or C.device != A.device:
             raise ValueError(f"C must be a ({m}, {n}) float32 or bfloat16 tensor on {A.device}")
     return _launch_gemm(A, a_fmt, a_pd, A_scale, B, b_fmt, b_pd, B_scale, C, accumulate=accumulate,
-                        kernel=kernel, block=32, split_k=split_k)
+                        kernel=kernel, block=32, split_k=split_k, static_scratch=static_scratch)
 
 
 def grouped_block_scaled_matmul(As, A_scales, Bs, B_scales, *, out_dtype: torch.dtype = torch.float32,

@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define MXGEMM_VERSION 101
+#define MXGEMM_VERSION 102
 
 /* Exported symbols (the library is built with hidden default visibility). */
 #if defined(__GNUC__)
@@ -144,6 +144,25 @@ MX_API int64_t mx_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, const mx
 MX_API int mx_gemm(const mx_tensor* A, const mx_tensor* A_scale, const mx_tensor* B,
             const mx_tensor* B_scale, mx_tensor* C, const mx_gemm_opts* opts, void* workspace,
             int64_t workspace_bytes, void* stream);
+
+/*
+ * mx_gemm for callers that cannot allocate or hand over device scratch: code running under HIP-graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its launcher needs no
+ * scratch; cext/tile_kernel.cpp:3874-3919 only launches).  Same operands, options, results and errors as
+ * mx_gemm, without the workspace arguments: the scale re-layout (and the split-K partial products) go to a
+ * buffer of MX_STATIC_SCRATCH_BYTES inside the library's own device image, one per GPU, held until the process
+ * ends.  Calls no hipMalloc / hipFree or any allocating routine.  A problem whose mx_gemm_workspace_bytes()
+ * exceeds MX_STATIC_SCRATCH_BYTES is refused with MX_ERR_WORKSPACE (8 MiB covers M*K + N*K <= 128 Mi elements,
+ * e.g. 16384 x 16384 x 4096; use mx_gemm beyond that).  Every call on a GPU shares that GPU's buffer, which
+ * keeps the previous call's contents; nothing in it has to start at zero (each call rewrites all it reads).
+ * Calls on one stream are ordered; calls that overlap on one GPU (several streams or host threads) race.
+ * The buffer's address is resolved on the first call on a device, or by mx_device_check(): make one of the
+ * two, and one warm-up call per kernel, before a capture begins.
+ */
+#define MX_STATIC_SCRATCH_BYTES (8 * 1024 * 1024)
+MX_API int64_t mx_static_scratch_bytes(void);
+MX_API int mx_gemm_static(const mx_tensor* A, const mx_tensor* A_scale, const mx_tensor* B,
+                   const mx_tensor* B_scale, mx_tensor* C, const mx_gemm_opts* opts, void* stream);
 
 /*
  * A list of independent block-scaled products C[i] = A[i] x B[i] (problem sizes may all differ), the
