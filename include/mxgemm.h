@@ -92,7 +92,10 @@ enum {
   MX_KERNEL_MFMA_256x256 = 3, /* 256x256 macro tile, 8 waves                                    */
   MX_KERNEL_MFMA_256x256_W4 = 4, /* 256x256 macro tile, 4 waves                                 */
   MX_KERNEL_DECODE = 5,       /* skinny-M (M <= 32) weight-streaming kernel                     */
-  MX_KERNEL_MFMA_PINGPONG = 6 /* 256x256 macro tile, two 4-wave teams alternating LDS/MFMA phases */
+  MX_KERNEL_MFMA_PINGPONG = 6, /* 256x256 macro tile, two 4-wave teams alternating LDS/MFMA phases,
+                                 v_mfma_scale_f32_16x16x128_f8f6f4                                */
+  MX_KERNEL_MFMA_PINGPONG32 = 7 /* the same schedule on v_mfma_scale_f32_32x32x64_f8f6f4; 8-bit
+                                 element formats only                                             */
 };
 
 typedef struct mx_gemm_opts {

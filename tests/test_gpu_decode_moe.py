@@ -94,7 +94,7 @@ def _moe_case(T, K, N, E, topk, seed, dev, w_std=0.1):
 
 
 @pytest.mark.parametrize("kernel,tile", [("generic", 16), ("generic", 128), ("mfma128", 128), ("mfma128", 256),
-                                         ("mfma256", 256), ("mfma256w4", 256), ("pingpong", 256), ("auto", 128), ("auto", 256)])
+                                         ("mfma256", 256), ("mfma256w4", 256), ("pingpong", 256), ("pingpong32", 256), ("auto", 128), ("auto", 256)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=str)
 def test_grouped_gemm_sample_shape(ct, dev, kernel, tile, out_dtype):
     """samples/MoE.py:420-462 shape: 48 tokens, hidden 512, 64 experts, top-8; N = 1024."""
@@ -124,7 +124,7 @@ def test_decode_two_halves_accumulate(ct, dev, K, x_fmt):
         assert O.rel_fro(acc.float().cpu(), ref + z.float()) <= tol
 
 
-@pytest.mark.parametrize("kernel", ["generic", "mfma128", "mfma256", "pingpong"])
+@pytest.mark.parametrize("kernel", ["generic", "mfma128", "mfma256", "pingpong", "pingpong32"])
 def test_grouped_gemm_routed_weight_replicas1_and_padded_ids(ct, dev, kernel):
     """Second GEMM of the sample: replicas = 1, rows multiplied by the routed weight
     (test/kernels/fused_moe.py:75-77); index arrays left at their worst-case length."""

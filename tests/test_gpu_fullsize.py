@@ -37,6 +37,13 @@ def test_square_8192_properties(ct, dev, fmt):
     # same K order: bit-identical
     c_ref = ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, out_dtype=torch.bfloat16, kernel="mfma256", **kw)
     assert torch.equal(c.view(torch.int16), c_ref.view(torch.int16))
+    c_32 = None
+    if fmt == O.E4M3:
+        # the 32x32x64-instruction kernel sums the products of a K block in another order inside the instruction:
+        # not bit-identical, but within a few bf16 roundings of the other kernels everywhere
+        c_32 = ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, out_dtype=torch.bfloat16, kernel="pingpong32", **kw)
+        assert O.rel_fro(c_32.float(), c_ref.float()) < 2e-3
+        assert bool(((c_32.float() - c_ref.float()).abs() <= 2.0 ** -6 * c_ref.float().abs() + 0.5).all())
 
     # doubling every A scale (E8M0 byte + 1) doubles the result exactly
     a_s2 = (a_s.view(torch.uint8) + 1).view(torch.float8_e8m0fnu)
@@ -56,6 +63,8 @@ def test_square_8192_properties(ct, dev, fmt):
     rows = torch.from_numpy(np.random.default_rng(7).choice(M, 64, replace=False))
     ref = a[rows].float() @ b.float().T
     assert O.rel_fro(c[rows.to(dev)].float().cpu(), ref) < 8e-3
+    if c_32 is not None:
+        assert O.rel_fro(c_32[rows.to(dev)].float().cpu(), ref) < 8e-3
 
 
 def test_decode_shape_properties(ct, dev):
