@@ -107,6 +107,9 @@ int launch_gemm_pingpong(const GemmArgs& g, hipStream_t stream);
 // the 32x32x64-instruction variant: 8-bit element formats only
 bool pingpong32_supports(int a_fmt, int b_fmt);
 int launch_gemm_pingpong32(const GemmArgs& g, hipStream_t stream);
+// persistent four-wave kernel (128 x 128 per wave): plain products of 8-bit operands, K >= 384
+bool gemm_w4_supports(const GemmArgs& g);
+int launch_gemm_w4(const GemmArgs& g, hipStream_t stream);
 // C[m, n] (+)= sum over `splits` fp32 partials [splits][M][N]; C fp32 or bf16 with row pitch ldc
 int launch_splitk_reduce(const float* partials, int splits, int64_t M, int64_t N, void* C, int64_t ldc,
                          int c_dtype, int accumulate, hipStream_t stream);

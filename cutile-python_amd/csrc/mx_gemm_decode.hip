@@ -340,54 +340,19 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
     const uint32_t xoff = (uint32_t)(m * d.ldx + q * SPW * 128 + gq * 16);
     const uint32_t xsoff = (uint32_t)(m * d.ldxs + q * SPW * 4);
     v4i xsraw[SPW / 4];
-#ifndef DEC_ORDER
-#define DEC_ORDER 0
-#endif
-    auto load_x = [&](int s) {
-#ifdef DEC_NOX
-      xf[s] = (v8i){s, 1, 2, 3, 4, 5, 6, 7};
-#else
+#pragma unroll
+    for (int s = 0; s < SPW; ++s) {
       const v4i lo = __builtin_amdgcn_raw_buffer_load_b128(rsX, xoff, s * 128, 0);
       const v4i hi = __builtin_amdgcn_raw_buffer_load_b128(rsX, xoff, s * 128 + 64, 0);
       xf[s] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-#endif
-    };
-    if (DEC_ORDER == 1 || DEC_ORDER == 2) { issue(t_first, 0); __builtin_amdgcn_sched_barrier(0); }
-    if (DEC_ORDER == 2) { if (t_count > 1) issue(t_first + G, 1); __builtin_amdgcn_sched_barrier(0); }
-#ifdef DEC_XROT
-    // the CUs of an XCD start their walk over the K-steps at different places
-    switch ((blockIdx.x >> 3) & 3) {
-      case 0:
-#pragma unroll
-        for (int s = 0; s < SPW; ++s) load_x(s);
-        break;
-      case 1:
-#pragma unroll
-        for (int s = 0; s < SPW; ++s) load_x((s + SPW / 4) % SPW);
-        break;
-      case 2:
-#pragma unroll
-        for (int s = 0; s < SPW; ++s) load_x((s + SPW / 2) % SPW);
-        break;
-      default:
-#pragma unroll
-        for (int s = 0; s < SPW; ++s) load_x((s + 3 * SPW / 4) % SPW);
-        break;
     }
-#else
-#pragma unroll
-    for (int s = 0; s < SPW; ++s) {
-      load_x(s);
-      if (DEC_ORDER == 3 && s == SPW / 2 - 1) { __builtin_amdgcn_sched_barrier(0); issue(t_first, 0); __builtin_amdgcn_sched_barrier(0); }
-    }
-#endif
 #pragma unroll
     for (int u = 0; u < SPW / 4; ++u) {
       xsraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rsXs, xsoff, u * 16, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (DEC_ORDER == 0) issue(t_first, 0);
-    if (DEC_ORDER != 2) { if (t_count > 1) issue(t_first + G, 1); }
+    issue(t_first, 0);
+    if (t_count > 1) issue(t_first + G, 1);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < SPW / 4; ++u) {
@@ -440,7 +405,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
     // that waves 0 and 1 issued after it is younger still, so they wait for the first load of tile i + 1 as
     // well -- measured: allowing for that store changes nothing, and counting it exactly would depend on
     // which form of the epilogue ran) ...
-    if (i + 1 < t_count && !(DEC_ORDER == 2 && i == 0)) {
+    if (i + 1 < t_count) {
       if (with_scales) __builtin_amdgcn_s_waitcnt(0x0F70 | (Cf::WIW + 1));
       else __builtin_amdgcn_s_waitcnt(0x0F70 | Cf::WIW);
     } else {

@@ -316,6 +316,7 @@ int launch_gemm_mfma(const GemmArgs& g, int kernel_id, hipStream_t stream) {
     case MX_KERNEL_MFMA_256x256_W4: return launch_fmt<256, 256, 2, 2>(g, stream);
     case MX_KERNEL_MFMA_PINGPONG: return launch_gemm_pingpong(g, stream);
     case MX_KERNEL_MFMA_PINGPONG32: return launch_gemm_pingpong32(g, stream);
+    case MX_KERNEL_MFMA_W4_PERSISTENT: return launch_gemm_w4(g, stream);
   }
   return set_error(MX_ERR_INVALID, "unknown MFMA kernel id %d", kernel_id);
 }

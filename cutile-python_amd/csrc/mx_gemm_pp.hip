@@ -272,9 +272,6 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   issue_b(0, 0);
   issue_a(1, 1);
   issue_b(1, 1);
-#pragma unroll
-  for (int u = 0; u < 2; ++u) sa[u] = As4[as_nxt[u]];
-  load_b_scales(bs_nxt);
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_barrier" ::: "memory");
@@ -288,6 +285,16 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     const int s = Q * SPQ + t0 / C::KSUB;
     if (s >= nstages) return;
     // =============================== memory phase ==================================================
+    if constexpr (t0 == 0) {
+      // Scales of this K-quad, first in the queue of this memory phase: they have the whole phase to arrive, and
+      // the MFMA phase holds no vector-memory instruction at all.  (Issued at the end of the previous quad's last
+      // MFMA phase instead, they met the other team's DMA burst in the address unit and held this team's arrival
+      // at the barrier: 2 % slower on MXFP8, 1 % on MXFP4.)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) sa[u] = As4[as_cur[u] + Q * 64];
+      load_b_scales(bs_cur + Q * 64);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     if constexpr (t0 == 0) {
       if (s == 0 && lid != walk.first) {
         // the previous tile's output leaves while the other team is in its MFMA phase
@@ -325,9 +332,8 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
       issue_b(sl_eff, bbuf);
-      // everything older than this phase's loads has landed: A and B of stage s + 1
-      // (the scale loads issued at the end of the previous quad are younger than those and may stay in
-      // flight; the MFMA phase waits for them)
+      // everything older than this phase's loads has landed: A and B of stage s + 1 (the scale loads issued
+      // at the start of this phase are younger than those and may stay in flight; the MFMA phase waits for them)
       constexpr int younger = (t0 == 0) ? P::SCALE_LOADS : 0;
       __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL + BL + younger));
     }
@@ -371,22 +377,11 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       if (ip + EARLY < 8) read_pair(ip + EARLY);
       mfma_pair(ip);
     }
-    constexpr bool last_of_quad = (t0 + C::KSUB == 4);
-    if constexpr (last_of_quad) {
-      // scales of the next K-quad (quad 0 of the tile being fetched after the last quad); they travel
-      // during the barrier and the next memory phase
-      const bool more = Q + 1 < KQ;
-      const int Qk = more ? Q + 1 : 0;
-#pragma unroll
-      for (int u = 0; u < 2; ++u) sa[u] = As4[(more ? as_cur[u] : as_nxt[u]) + Qk * 64];
-      load_b_scales((more ? bs_cur : bs_nxt) + Qk * 64);
-    }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (TEAM == 0) {
-      // A of stage s + 1 (issued one stage ago) must have landed; A of stage s + 2 and the scale
-      // loads just issued may stay in flight
-      __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL + (last_of_quad ? P::SCALE_LOADS : 0)));
+      // A of stage s + 1 (issued one stage ago) must have landed; A of stage s + 2 may stay in flight
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL));
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);

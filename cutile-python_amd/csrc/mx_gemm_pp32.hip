@@ -294,7 +294,6 @@ __device__ __forceinline__ void pp32_body(const GemmArgs& g, lds_u8* const smem,
   issue_b(0, 0);
   issue_a(1, 1);
   issue_b(1, 1);
-  load_scales(as_nxt, bs_nxt, 0);
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_barrier" ::: "memory");
@@ -309,6 +308,8 @@ __device__ __forceinline__ void pp32_body(const GemmArgs& g, lds_u8* const smem,
     if (s >= nstages) return;
     // =============================== memory phase ==================================================
     if constexpr (t0 == 0) {
+      load_scales(as_cur, bs_cur, Q);   // first in this memory phase's queue (see mx_gemm_pp.hip)
+      __builtin_amdgcn_sched_barrier(0);
       if (s == 0 && lid != walk.first) {
         int plid = lid - walk.step;
         asm volatile("" : "+s"(plid));
@@ -361,15 +362,10 @@ __device__ __forceinline__ void pp32_body(const GemmArgs& g, lds_u8* const smem,
           acc[I][J] = mfma32<C::BF, C::AF, t0>(bf[J][u], af[I][u], acc[I][J], sb[J][u], sa[I][u]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    constexpr bool last_of_quad = (t0 == 3);
-    if constexpr (last_of_quad) {
-      const bool more = Q + 1 < KQ;
-      load_scales(more ? as_cur : as_nxt, more ? bs_cur : bs_nxt, more ? Q + 1 : 0);
-    }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (TEAM == 0) {
-      __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL + (last_of_quad ? SCALE_LOADS : 0)));
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL));
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);

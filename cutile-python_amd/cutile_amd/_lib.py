@@ -24,11 +24,13 @@ MX_KERNEL_AUTO, MX_KERNEL_GENERIC = 0, 1
 MX_KERNEL_MFMA_128x128, MX_KERNEL_MFMA_256x256, MX_KERNEL_MFMA_256x256_W4, MX_KERNEL_DECODE = 2, 3, 4, 5
 MX_KERNEL_MFMA_PINGPONG = 6
 MX_KERNEL_MFMA_PINGPONG32 = 7
+MX_KERNEL_MFMA_W4_PERSISTENT = 8
 
 KERNELS = {
     "auto": MX_KERNEL_AUTO, "generic": MX_KERNEL_GENERIC, "mfma128": MX_KERNEL_MFMA_128x128,
     "mfma256": MX_KERNEL_MFMA_256x256, "mfma256w4": MX_KERNEL_MFMA_256x256_W4, "decode": MX_KERNEL_DECODE,
     "pingpong": MX_KERNEL_MFMA_PINGPONG, "pingpong32": MX_KERNEL_MFMA_PINGPONG32,
+    "w4p": MX_KERNEL_MFMA_W4_PERSISTENT,
 }
 
 

@@ -94,8 +94,11 @@ enum {
   MX_KERNEL_DECODE = 5,       /* skinny-M (M <= 32) weight-streaming kernel                     */
   MX_KERNEL_MFMA_PINGPONG = 6, /* 256x256 macro tile, two 4-wave teams alternating LDS/MFMA phases,
                                  v_mfma_scale_f32_16x16x128_f8f6f4                                */
-  MX_KERNEL_MFMA_PINGPONG32 = 7 /* the same schedule on v_mfma_scale_f32_32x32x64_f8f6f4; 8-bit
+  MX_KERNEL_MFMA_PINGPONG32 = 7, /* the same schedule on v_mfma_scale_f32_32x32x64_f8f6f4; 8-bit
                                  element formats only                                             */
+  MX_KERNEL_MFMA_W4_PERSISTENT = 8 /* 256x256 macro tile, four waves of 128x128 (one per SIMD, 512
+                                 registers), self-pipelined, 32x32x64 instruction; plain products of
+                                 8-bit operands with K >= 384                                     */
 };
 
 typedef struct mx_gemm_opts {

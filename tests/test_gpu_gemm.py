@@ -239,3 +239,30 @@ def test_split_k_rejects_impossible_requests(ct, dev):
         _run(ct, a, b, split_k=2)          # 1536 is not a multiple of 1024
     with pytest.raises(Exception, match="one-tile MFMA kernels"):
         _run(ct, a, b, split_k=3, kernel="generic")
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 512), (512, 768, 1024), (300, 520, 384), (256, 256, 416), (3072, 3072, 1024),
+                                   (1, 1, 384), (777, 1030, 4096)])
+def test_four_wave_persistent_kernel(ct, dev, fmt, M, N, K):
+    """The four-wave kernel (128 x 128 per wave, 32x32x64 instruction, five-buffer half-stage ring): aligned and
+    ragged shapes, a K that ends inside a half-stage and inside a K-quad, more tiles than workgroups' first
+    round, fp32 and bf16 output with and without accumulation."""
+    a, b = randn_operand(M, K, fmt, 31, dev), randn_operand(N, K, fmt, 32, dev)
+    ref = oracle_matmul(a, b)
+    for out_dtype in (torch.float32, torch.bfloat16):
+        c = _run(ct, a, b, out_dtype=out_dtype, kernel="w4p")
+        _check(c, ref, out_dtype, f"w4p {fmt} {M}x{N}x{K} {out_dtype}")
+    z = torch.randn((M, N), generator=torch.Generator().manual_seed(33))
+    acc = z.to(dev)
+    _run(ct, a, b, C=acc, accumulate=True, kernel="w4p")
+    _check(acc, ref + z, torch.float32, "w4p accumulate")
+
+
+def test_four_wave_kernel_rejects_what_it_cannot_run(ct, dev):
+    a, b = randn_operand(256, 256, O.E4M3, 1, dev), randn_operand(256, 256, O.E4M3, 2, dev)
+    with pytest.raises(ct.TileTypeError, match="K >= 384"):
+        _run(ct, a, b, kernel="w4p")
+    a4, b4 = randn_operand(256, 512, O.E2M1, 1, dev), randn_operand(256, 512, O.E2M1, 2, dev)
+    with pytest.raises(ct.TileTypeError, match="8-bit"):
+        _run(ct, a4, b4, kernel="w4p")
