@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the block-scaled (MX) matmul path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2|c3|c4|c5] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,c3,c4,c5,r4096] [--kernel NAME] [--no-cpu]
 
 A "step" is one call of the hot path -- block_scaled_matmul(A, A_scale, B, B_scale, out_dtype=bf16) with
 the reference's tensor layouts (plain (M, K/32) / (K/32, N) E8M0 scales, so the per-call scale re-layout
@@ -11,8 +11,13 @@ single-GPU configurations of the metric (MXFP4 8192^3, the M = 32 decode GEMM, t
 timed the same way and reported under "extra".
 
 Prints ONE JSON line.  `roofline` describes the dominant kernel of the headline workload: algorithmic
-flops per launch divided by the kernel's average duration, measured with HIP events on the launch stream
-around launches of the GEMM kernel alone (scales pre-packed, so no other kernel runs in that region).
+flops per launch divided by the kernel's average duration, measured with one pair of HIP events per launch on
+the launch stream around launches of the GEMM kernel alone (scales pre-packed, so no other kernel runs between
+the events).  The samples follow the reference tuner's protocol (src/cuda/tile/tune/_tune.py:339-395): batches
+of 5 until the 95 % confidence half-width is below 1 % of the mean (or 0.5 us), at least 20 samples; n, mean,
+min and the half-width are reported.  Every configuration under `extra` carries the same kind of object.
+`traffic` (HBM bytes per launch) comes from rocprofv3 --pmc runs of this file; it is read from the summary
+under profiles/ so that it cannot outlive the kernel it was measured on (null if no figure is kept there).
 `cpu_baseline` times the oracle's dequantize + fp32 matmul on this host's cores on an N-slice of the same
 workload.  Operand sets are rotated so that no launch finds its inputs in L2 / Infinity Cache.  Every timed
 region is preceded by an untimed settle period of the same steps (see _settle) and the W warm-up steps.
@@ -23,6 +28,7 @@ import argparse
 import json
 import os
 import pathlib
+import re
 import sys
 import time
 
@@ -35,10 +41,7 @@ import torch  # noqa: E402
 
 PEAK_TFLOPS = {"mxfp8": 5033.0, "mxfp4": 10066.0}   # MI355X dense MFMA peaks (vendor figures)
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the headline GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# `bench.py --only c2 --calib-copy`, each scaled by what the same counter reads for the 256 MiB copy kernel
-# (summary under profiles/): 405775 KiB x 2.0 + 132002 KiB x 1.0
-C2_HBM_TRAFFIC_BYTES = 943552 * 1024
+PROFILE_TRAFFIC = ROOT / "profiles" / "hbm_traffic_pmc.md"
 METRIC = "MX GEMM TFLOP/s (+% MFMA peak) 8192^3 MXFP8/MXFP4; GB/s at M=32 decode"
 
 
@@ -93,6 +96,57 @@ def _time_events(fn, steps, warmup):
     return start.elapsed_time(stop) * 1e-3 / steps
 
 
+class Welford:
+    """Running mean / variance of per-launch durations and the stopping rule of the reference's tuner
+    (src/cuda/tile/tune/_tune.py:339-395)."""
+
+    def __init__(self):
+        self.n, self.mean, self.m2, self.min, self.max = 0, 0.0, 0.0, float("inf"), 0.0
+
+    def add(self, x):
+        self.n += 1
+        d = x - self.mean
+        self.mean += d / self.n
+        self.m2 += d * (x - self.mean)
+        self.min, self.max = min(self.min, x), max(self.max, x)
+
+    @property
+    def margin(self):   # 95 % confidence half-width of the mean
+        return 1.96 * (self.m2 / (self.n - 1) / self.n) ** 0.5 if self.n > 1 else float("inf")
+
+    def converged(self, min_samples):
+        return self.n >= min_samples and (self.margin <= 0.01 * self.mean or self.margin <= 0.5 or self.n >= 1000
+                                          or self.mean * self.n > 5e6)
+
+    def stats(self):
+        return {"n": self.n, "mean_us": self.mean, "min_us": self.min, "max_us": self.max, "ci95_us": self.margin}
+
+
+def measure(batch_fn, min_samples=20, batch=5):
+    """batch_fn(k) -> k per-launch durations in microseconds (it does its own warm-up on the first call)."""
+    w = Welford()
+    while not w.converged(min_samples):
+        for t in batch_fn(batch):
+            w.add(t)
+    return w
+
+
+def profile_traffic(tag):
+    """HBM bytes per launch of configuration `tag`, from the line `traffic_bytes[tag] = N` of the rocprofv3
+    summary under profiles/ (None if there is none)."""
+    try:
+        m = re.search(rf"traffic_bytes\[{tag}\]\s*=\s*(\d+)", PROFILE_TRAFFIC.read_text())
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def roofline(bound, achieved, peak, unit, tag, kernel, w, work):
+    return {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
+            "traffic": profile_traffic(tag), "kernel": kernel, "kernel_ms": w.mean * 1e-3,
+            ("flops_per_launch" if bound == "mfma" else "bytes_per_launch"): work, **w.stats()}
+
+
 def _quantized(ct, rows, K, fmt, seed, dev, dist, std=1.0, cpu_seeded=True):
     """(storage, scale) on the device.  The first operand set of every workload comes from a seeded CPU
     generator (the workload definition); rotation copies are drawn on the device."""
@@ -127,7 +181,30 @@ def _check_rows(O, c, ref, rows, tol, what):
     return err
 
 
-def bench_gemm(ct, O, dev, M, N, K, fmt, dist, steps, warmup, check, nsets=3):
+def _events_batch(fn, settle=True):
+    """batch_fn for `measure`: each call of fn(i) between its own pair of events on the current stream."""
+    state = {"i": 0, "warm": False}
+
+    def batch(k):
+        if not state["warm"]:
+            if settle:
+                _settle(fn)
+            for _ in range(3):
+                fn(state["i"])
+                state["i"] += 1
+            state["warm"] = True
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(k)]
+        for e0, e1 in ev:
+            e0.record()
+            fn(state["i"])
+            e1.record()
+            state["i"] += 1
+        _sync()
+        return [e0.elapsed_time(e1) * 1e3 for e0, e1 in ev]
+    return batch
+
+
+def bench_gemm(ct, O, dev, M, N, K, fmt, dist, steps, warmup, check, kernel="auto", nsets=3):
     """Square / large GEMM configurations (MXFP8 or MXFP4, bf16 out)."""
     tfmt = torch.float8_e4m3fn if fmt == O.E4M3 else "e2m1"
     kw = {} if fmt == O.E4M3 else {"a_format": "e2m1", "b_format": "e2m1"}
@@ -139,26 +216,30 @@ def bench_gemm(ct, O, dev, M, N, K, fmt, dist, steps, warmup, check, nsets=3):
     err = None
     if check:
         a_q, a_s, b_q, b_s, c = sets[0]
-        ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, C=c, **kw)
+        ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, C=c, kernel=kernel, **kw)
         rows = torch.arange(0, M, max(1, M // 32))[:32]
         err = _check_rows(O, c, _oracle_rows(O, a_q, a_s, b_q, b_s, rows, fmt, fmt), rows, 8e-3, f"{fmt} {M}x{N}x{K}")
 
     def step(i):
         a_q, a_s, b_q, b_s, c = sets[i % nsets]
-        ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, C=c, **kw)
+        ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, C=c, kernel=kernel, **kw)
 
     t_step = _time_wall(step, steps, warmup)
-    packed = [(ct.pack_scales(s[1]), ct.pack_scales(s[3])) for s in sets]
+    # kernel alone: scales pre-packed, one pair of HIP events per launch recorded by the library's own timing
+    # entry point (mx_bench_gemm) on the launch stream, operand sets rotated
+    packed = [(s[0], ct.pack_scales(s[1]), s[2].T, ct.pack_scales(s[3]), s[4]) for s in sets]
+    state = {"warm": False}
 
-    def kernel_only(i):
-        a_q, _, b_q, _, c = sets[i % nsets]
-        pa, pb = packed[i % nsets]
-        ct.block_scaled_matmul(a_q, pa, b_q.T, pb, C=c, **kw)
+    def batch(k):
+        if not state["warm"]:
+            _settle(lambda i: ct.block_scaled_matmul(*packed[i % nsets][:4], C=packed[i % nsets][4], kernel=kernel, **kw))
+            state["warm"] = True
+        return [t * 1e3 for t in ct.bench_block_scaled_matmul(packed, warmup=3, iters=k, kernel=kernel, **kw)]
 
-    t_kernel = _time_events(kernel_only, steps, warmup)
+    w = measure(batch, batch=10)
     flops = 2.0 * M * N * K
-    return {"ms_per_step": t_step * 1e3, "tflops": flops / t_step * 1e-12, "kernel_ms": t_kernel * 1e3,
-            "kernel_tflops": flops / t_kernel * 1e-12, "rel_fro_vs_oracle": err, "flops": flops, "sets": sets}
+    return {"ms_per_step": t_step * 1e3, "tflops": flops / t_step * 1e-12, "kernel": w,
+            "kernel_tflops": flops / (w.mean * 1e-6) * 1e-12, "rel_fro_vs_oracle": err, "flops": flops, "sets": sets}
 
 
 def vendor_scaled_mm(sets, steps, warmup):
@@ -202,18 +283,13 @@ def bench_recorded_4096(ct, O, dev, steps, warmup, check, nsets=4):
         ct.block_scaled_matmul(a_q, a_sw, b_q.T, b_sw, C=c)
 
     t_call = _time_events(step, steps, warmup)
-    packed = [(ct.pack_scales(s[1]), ct.pack_scales(s[3])) for s in sets]
-
-    def kernel_only(i):
-        a_q, _, b_q, _, _, _, c = sets[i % nsets]
-        pa, pb = packed[i % nsets]
-        ct.block_scaled_matmul(a_q, pa, b_q.T, pb, C=c)
-
-    t_kernel = _time_events(kernel_only, steps, warmup)
+    packed = [(s[0], ct.pack_scales(s[1]), s[2].T, ct.pack_scales(s[3]), s[6]) for s in sets]
+    w = measure(lambda k: [t * 1e3 for t in ct.bench_block_scaled_matmul(packed, warmup=3, iters=k)], batch=10)
     flops = 2.0 * M * N * K
     return {"call_us_incl_scale_relayout": t_call * 1e6, "tflops": flops / t_call * 1e-12,
-            "gemm_kernel_us": t_kernel * 1e6, "gemm_kernel_tflops": flops / t_kernel * 1e-12,
-            "reference_recorded_us_b200": 71.379, "rel_fro_vs_oracle": err}
+            "gemm_kernel_us": w.mean, "gemm_kernel_tflops": flops / w.mean * 1e-6, **w.stats(),
+            "reference_recorded_us_b200": 71.379, "reference_recorded_ci_us_b200": 0.294,
+            "rel_fro_vs_oracle": err}
 
 
 def bench_decode(ct, O, dev, steps, warmup, check, nsets=8):
@@ -243,14 +319,15 @@ def bench_decode(ct, O, dev, steps, warmup, check, nsets=8):
     with torch.cuda.graph(graph):
         for i in range(nsets):
             step(i)
-    reps = max(1, (steps + nsets - 1) // nsets)
-    t = _time_events(lambda i: graph.replay(), reps, 2) / nsets
+    # one sample = one replay (nsets launches back to back on the stream) between a pair of events, / nsets
+    rb = _events_batch(lambda i: graph.replay())
+    w = measure(lambda k: [t / nsets for t in rb(k)])
     nbytes = M * K + M * K // 32 + N * K // 2 + N * K // 32 + M * N * 2     # 126 885 888
-    return {"ms_per_step": t_wall * 1e3, "kernel_ms": t * 1e3, "gbs": nbytes / t * 1e-9,
+    return {"ms_per_step": t_wall * 1e3, "kernel": w, "gbs": nbytes / (w.mean * 1e-6) * 1e-9,
             "gbs_wall": nbytes / t_wall * 1e-9, "bytes": nbytes, "rel_fro_vs_oracle": err}
 
 
-def bench_moe(ct, O, dev, steps, warmup, check):
+def bench_moe(ct, O, dev, steps, warmup, check, full_forward=True):
     """MoE grouped MXFP8 GEMM: 4096 tokens, hidden 4096, 8 experts x 14336, top-2 (8192 routed rows)."""
     T, K, N, E, topk, tile = 4096, 4096, 14336, 8, 2, 256
     x_q, x_s = _quantized(ct, T, K, torch.float8_e4m3fn, 3001, dev, "randn")
@@ -291,10 +368,15 @@ def bench_moe(ct, O, dev, steps, warmup, check):
     def kernel_mostly(i):
         ct.invoke_fused_moe_scaled(x_q, x_s, W, pW, C, None, sid, eid, False, topk, tile)
 
-    t_k = _time_events(kernel_mostly, steps, warmup)
+    # the grouped GEMM kernel with the expert scales pre-packed: the only other kernel between the events is the
+    # re-layout of the (gathered) activation scales, 0.5 MiB
+    w = measure(_events_batch(kernel_mostly))
     flops = 2.0 * T * topk * K * N
-    out = {"ms_per_step": t_step * 1e3, "tflops": flops / t_step * 1e-12, "kernel_ms": t_k * 1e3,
-           "kernel_tflops": flops / t_k * 1e-12, "rel_fro_vs_oracle": err, "padded_rows": int(sid.numel())}
+    out = {"ms_per_step": t_step * 1e3, "tflops": flops / t_step * 1e-12, "kernel": w,
+           "kernel_tflops": flops / (w.mean * 1e-6) * 1e-12, "rel_fro_vs_oracle": err, "padded_rows": int(sid.numel()),
+           "flops": flops}
+    if not full_forward:
+        return out
     # Informational: the whole block-scaled MoE forward the up-projection belongs to (alignment, gate+up GEMM,
     # SiLU * up with re-quantisation, down GEMM with the routed weights, sum over the top-k copies), N = 2 F.
     F = N // 2
@@ -359,6 +441,12 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c5,r4096 (default: all)")
+    ap.add_argument("--kernel", default="auto",
+                    help="kernel of the square GEMM legs: auto, pingpong, pingpong32, w4p, mfma256, mfma256w4, mfma128 "
+                         "(the counter comparisons under profiles/ are runs of this file with this option)")
+    ap.add_argument("--no-moe-forward", action="store_true",
+                    help="c5: only the up-projection grouped GEMM (a kernel trace of the run then holds one shape of "
+                         "the grouped kernel), not the whole MoE forward")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the correctness check before timing")
     ap.add_argument("--settle-ms", type=float, default=SETTLE_S * 1e3,
@@ -389,49 +477,54 @@ def main():
         del src, dst
     want = set(filter(None, a.only.split(","))) or {"c2", "c3", "c4", "c5", "r4096"}
     check = not a.no_check
+    kname = {"auto": "gemm_pp_kernel", "pingpong": "gemm_pp_kernel", "pingpong32": "gemm_pp32_kernel",
+             "w4p": "gemm_w4_kernel", "mfma256": "gemm_kernel<256x256,8 waves>", "mfma256w4": "gemm_kernel<256x256,4 waves>",
+             "mfma128": "gemm_kernel<128x128>"}.get(a.kernel, a.kernel)
     extra = {}
     if "c4" in want:
-        r = bench_gemm(ct, O, dev, 8192, 8192, 8192, O.E2M1, "uniform6", a.steps, a.warmup, check)
-        r.pop("sets")
+        r = bench_gemm(ct, O, dev, 8192, 8192, 8192, O.E2M1, "uniform6", a.steps, a.warmup, check,
+                       kernel=a.kernel if a.kernel != "pingpong32" and a.kernel != "w4p" else "auto")
         extra["c4_mxfp4_8192"] = {"tflops": r["tflops"], "ms_per_step": r["ms_per_step"],
-                                  "kernel_tflops": r["kernel_tflops"], "frac_of_mxfp4_peak": r["kernel_tflops"] / PEAK_TFLOPS["mxfp4"],
-                                  "rel_fro_vs_oracle": r["rel_fro_vs_oracle"]}
+                                  "rel_fro_vs_oracle": r["rel_fro_vs_oracle"],
+                                  "roofline": roofline("mfma", r["kernel_tflops"], PEAK_TFLOPS["mxfp4"], "TFLOP/s", "c4",
+                                                       "gemm_pp_kernel<Cfg<e2m1,e2m1,256,256,2,4>,bf16>", r["kernel"], r["flops"])}
+        del r
         torch.cuda.empty_cache()
     if "r4096" in want:
         extra["recorded_problem_mxfp8_4096_swizzled_fp32"] = bench_recorded_4096(ct, O, dev, a.steps, a.warmup, check)
         torch.cuda.empty_cache()
     if "c3" in want:
         r = bench_decode(ct, O, dev, max(a.steps, 50), a.warmup, check)
-        extra["c3_decode_m32"] = {"gbs": r["gbs"], "kernel_us": r["kernel_ms"] * 1e3, "gbs_wall_clock": r["gbs_wall"],
-                                  "frac_of_hbm_peak": r["gbs"] / PEAK_HBM_GBS, "bytes": r["bytes"],
-                                  "rel_fro_vs_oracle": r["rel_fro_vs_oracle"]}
+        extra["c3_decode_m32"] = {"gbs_wall_clock": r["gbs_wall"], "ms_per_step": r["ms_per_step"],
+                                  "rel_fro_vs_oracle": r["rel_fro_vs_oracle"],
+                                  "roofline": roofline("hbm", r["gbs"], PEAK_HBM_GBS, "GB/s", "c3",
+                                                       "decode2_kernel<e4m3,16,bf16>", r["kernel"], r["bytes"])}
         torch.cuda.empty_cache()
     if "c5" in want:
-        r = bench_moe(ct, O, dev, a.steps, a.warmup, check)
-        extra["c5_moe_grouped_mxfp8"] = {"tflops": r["tflops"], "ms_per_step": r["ms_per_step"],
-                                         "kernel_tflops": r["kernel_tflops"],
-                                         "frac_of_mxfp8_peak": r["kernel_tflops"] / PEAK_TFLOPS["mxfp8"],
-                                         "padded_rows": r["padded_rows"], "rel_fro_vs_oracle": r["rel_fro_vs_oracle"],
-                                         "full_forward_ms": r["full_forward_ms"],
-                                         "full_forward_tflops": r["full_forward_tflops"]}
+        r = bench_moe(ct, O, dev, a.steps, a.warmup, check, full_forward=not a.no_moe_forward)
+        e5 = {"tflops": r["tflops"], "ms_per_step": r["ms_per_step"], "padded_rows": r["padded_rows"],
+              "rel_fro_vs_oracle": r["rel_fro_vs_oracle"],
+              "roofline": roofline("mfma", r["kernel_tflops"], PEAK_TFLOPS["mxfp8"], "TFLOP/s", "c5",
+                                   "gemm_pp_kernel<Cfg<e4m3,e4m3,256,256,2,4>,bf16,grouped>", r["kernel"], r["flops"])}
+        if "full_forward_ms" in r:
+            e5["full_forward_ms"], e5["full_forward_tflops"] = r["full_forward_ms"], r["full_forward_tflops"]
+        extra["c5_moe_grouped_mxfp8"] = e5
         torch.cuda.empty_cache()
     out = {"metric": METRIC, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "mxfp8_e4m3 (e8m0 scales, fp32 accumulate, bf16 out)",
            "data": "synthetic", "settle_ms": SETTLE_S * 1e3, "extra": extra}
     if "c2" in want:
-        r = bench_gemm(ct, O, dev, 8192, 8192, 8192, O.E4M3, "randn", a.steps, a.warmup, check)
+        r = bench_gemm(ct, O, dev, 8192, 8192, 8192, O.E4M3, "randn", a.steps, a.warmup, check, kernel=a.kernel)
         out.update({
             "value": r["tflops"], "ms_per_step": r["ms_per_step"],
             "config": {"workload": "MXFP8 E4M3 x E4M3 block-scaled GEMM, M=N=K=8192, E8M0 scale per 32 along K "
                                    "(floor rule), A row-major MxK, B column-major KxN, fp32 accumulate, bf16 output; "
                                    "one step = one block_scaled_matmul call incl. scale re-layout",
-                       "M": 8192, "N": 8192, "K": 8192, "operand_sets_rotated": 3},
+                       "M": 8192, "N": 8192, "K": 8192, "operand_sets_rotated": 3, "kernel": a.kernel},
             "rel_fro_vs_oracle": r["rel_fro_vs_oracle"],
-            "roofline": {"bound": "mfma", "achieved": r["kernel_tflops"], "peak": PEAK_TFLOPS["mxfp8"],
-                         "unit": "TFLOP/s", "frac": r["kernel_tflops"] / PEAK_TFLOPS["mxfp8"],
-                         "traffic": C2_HBM_TRAFFIC_BYTES,
-                         "kernel": "gemm_pp_kernel<Cfg<e4m3,e4m3,256,256,2,4>,bf16>", "kernel_ms": r["kernel_ms"],
-                         "flops_per_launch": r["flops"]},
+            "roofline": roofline("mfma", r["kernel_tflops"], PEAK_TFLOPS["mxfp8"], "TFLOP/s",
+                                 "c2" if a.kernel in ("auto", "pingpong") else "c2_" + a.kernel,
+                                 f"{kname}<e4m3,e4m3,256x256,bf16>", r["kernel"], r["flops"]),
         })
         if not a.no_vendor:
             extra["context_torch_scaled_mm_mxfp8_8192"] = vendor_scaled_mm(r["sets"], a.steps, a.warmup)
