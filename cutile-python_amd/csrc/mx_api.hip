@@ -5,6 +5,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <vector>
 
 #include "mx_common.h"
 
@@ -224,8 +225,30 @@ int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t
   return launch_pack_scales(p, (hipStream_t)stream);
 }
 
+namespace {
+// What mx_gemm would launch for a problem that ends on the 128 x 128 one-tile kernel without split-K: the list
+// entry point collects these and runs them as one batched scale re-layout and one persistent GEMM launch.
+struct GemmPlan {
+  GemmArgs g;
+  PackArgs pa, pb;
+  bool pack_a, pack_b;
+};
+constexpr int kPlanNotSimple = 1;   // gemm_impl with a plan: the problem needs its own mx_gemm call
+
+int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const mx_tensor* Bs, mx_tensor* C,
+              const mx_gemm_opts* opts, void* workspace, int64_t workspace_bytes, void* stream, GemmPlan* plan);
+}  // namespace
+
 int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const mx_tensor* Bs, mx_tensor* C,
             const mx_gemm_opts* opts, void* workspace, int64_t workspace_bytes, void* stream) {
+  return gemm_impl(A, As, B, Bs, C, opts, workspace, workspace_bytes, stream, nullptr);
+}
+
+namespace {
+// mx_gemm; with `plan` nothing is launched: a problem of the simple kind is described in *plan (return MX_OK),
+// any other valid problem returns kPlanNotSimple
+int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const mx_tensor* Bs, mx_tensor* C,
+              const mx_gemm_opts* opts, void* workspace, int64_t workspace_bytes, void* stream, GemmPlan* plan) {
   const mx_gemm_opts& o = opts ? *opts : kDefaultOpts;
   if (int rc = check_tensor(A, "A", 2, 3)) return rc;
   if (int rc = check_tensor(B, "B", 2, 3)) return rc;
@@ -280,13 +303,14 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
       return set_error(MX_ERR_SHAPE, "B_scale shape is not compatible with B: expected [.., %lld, %lld]",
                        (long long)KB, (long long)N);
   }
-  if (M == 0 || N == 0) return MX_OK;
+  if (M == 0 || N == 0) return plan ? kPlanNotSimple : MX_OK;
 
   // ---- batched operands (test/test_mma_scaled.py:128-145): one 2-D product per batch entry, size-1
   // batches broadcast; stream order lets the entries share the workspace.  Layouts only the generic
   // kernel reads (block 16, E4M3 scales) keep its own batched launch. --------------------------------
   if (batched && o.kernel != MX_KERNEL_GENERIC && o.block_size == 32 && As->dtype == MX_E8M0 &&
       o.a_scale_layout == MX_SCALE_2D && o.b_scale_layout == MX_SCALE_2D) {
+    if (plan) return kPlanNotSimple;
     auto slice = [](const mx_tensor* t, int64_t b, int elem_bytes) {
       mx_tensor v = *t;
       if (t->ndim == 3) {
@@ -336,6 +360,7 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
       kernel != MX_KERNEL_MFMA_256x256_W4)
     return set_error(MX_ERR_LAYOUT, "split_k = %d is only available on the one-tile MFMA kernels (kernel %d chosen)",
                      o.split_k, kernel);
+  if (plan && kernel != MX_KERNEL_MFMA_128x128) return kPlanNotSimple;
   if (kernel == MX_KERNEL_GENERIC) {
     if (o.a_scale_layout == MX_SCALE_NATIVE || o.b_scale_layout == MX_SCALE_NATIVE)
       return set_error(MX_ERR_LAYOUT, "the generic kernel cannot read native-layout scales");
@@ -413,6 +438,7 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
       return set_error(MX_ERR_SHAPE, "split_k = %d needs K (%lld) to be a multiple of %d", o.split_k, (long long)K,
                        512 * o.split_k);
   }
+  if (S > 1 && plan) return kPlanNotSimple;
   if (S > 1) {
     // ---- split-K: the slices are a batch for the scale re-layout and a second grid dimension for the GEMM
     const int64_t Ks = K / S, kbs = Ks / 32;
@@ -458,10 +484,10 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
     if (int rc = make_pack_args(&t, o.b_scale_layout, N, K, ws, pb)) return rc;
     bs_native = (const uint32_t*)ws;
   }
-  if (pack_a || pack_b)   // one launch for both operands
-    if (int rc = launch_pack_scales_pair(pack_a ? &pa : nullptr, pack_b ? &pb : nullptr, (hipStream_t)stream)) return rc;
   if (((uintptr_t)as_native) % 16 != 0 || ((uintptr_t)bs_native) % 16 != 0)
     return set_error(MX_ERR_LAYOUT, "native scale buffers must be 16-byte aligned");
+  if (!plan && (pack_a || pack_b))   // one launch for both operands
+    if (int rc = launch_pack_scales_pair(pack_a ? &pa : nullptr, pack_b ? &pb : nullptr, (hipStream_t)stream)) return rc;
 
   GemmArgs g = {};
   g.A = (const uint8_t*)A->ptr; g.B = (const uint8_t*)B->ptr; g.As = as_native; g.Bs = bs_native; g.C = C->ptr;
@@ -470,8 +496,17 @@ int mx_gemm(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const m
   g.a_fmt = A->dtype; g.b_fmt = B->dtype; g.c_dtype = C->dtype; g.accumulate = o.accumulate;
   g.a_rows = M;
   g.replicas = 1;
+  if (plan) {
+    if ((pack_a && o.a_scale_layout != MX_SCALE_2D) || (pack_b && o.b_scale_layout != MX_SCALE_2D)) return kPlanNotSimple;
+    plan->g = g;
+    plan->pack_a = pack_a; plan->pack_b = pack_b;
+    if (pack_a) plan->pa = pa;
+    if (pack_b) plan->pb = pb;
+    return MX_OK;
+  }
   return launch_gemm_mfma(g, kernel, (hipStream_t)stream);
 }
+}  // namespace
 
 namespace {
 // logical (M, N, K) of a problem from its operand descriptors (FP4 operands count elements, not bytes)
@@ -505,12 +540,11 @@ int mx_gemm_static(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, 
 int64_t mx_gemm_list_workspace_bytes(int32_t count, const mx_tensor* A, const mx_tensor* B,
                                      const mx_gemm_opts* opts) {
   if (count <= 0 || !A || !B) return 0;
-  int64_t need = 0;
+  int64_t need = 0;   // every problem has its own slice: the problems of a list run side by side
   for (int32_t i = 0; i < count; ++i) {
     int64_t M, N, K;
     problem_dims(A[i], B[i], M, N, K);
-    const int64_t b = mx_gemm_workspace_bytes(M, N, K, opts);
-    need = b > need ? b : need;
+    need += round256(mx_gemm_workspace_bytes(M, N, K, opts));
   }
   return need;
 }
@@ -520,11 +554,67 @@ int mx_gemm_list(int32_t count, const mx_tensor* A, const mx_tensor* As, const m
   if (count < 0) return set_error(MX_ERR_INVALID, "mx_gemm_list: negative count");
   if (count == 0) return MX_OK;
   if (!A || !As || !B || !Bs || !C) return set_error(MX_ERR_INVALID, "mx_gemm_list: null descriptor array");
+  const int64_t need = mx_gemm_list_workspace_bytes(count, A, B, opts);
+  if (need > 0 && (!workspace || workspace_bytes < need))
+    return set_error(MX_ERR_WORKSPACE, "workspace of %lld bytes required, %lld given", (long long)need,
+                     (long long)workspace_bytes);
+  if (need > 0 && ((uintptr_t)workspace) % 256 != 0) return set_error(MX_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+
+  // Pass 1: validate everything and sort the problems: those that would run on the 128 x 128 one-tile kernel are
+  // collected (no launch), the others are remembered for a call of their own.  Nothing is enqueued if any problem
+  // is invalid.
+  struct Item { int32_t index; int64_t ws_off, ws_bytes; bool simple; GemmPlan plan; };
+  std::vector<Item> items;
+  items.reserve(count);
+  int64_t off = 0;
   for (int32_t i = 0; i < count; ++i) {
     int64_t M, N, K;
     problem_dims(A[i], B[i], M, N, K);
-    if (A[i].ndim == 2 && B[i].ndim == 2 && (M == 0 || N == 0)) continue;
-    const int rc = mx_gemm(&A[i], &As[i], &B[i], &Bs[i], &C[i], opts, workspace, workspace_bytes, stream);
+    const int64_t b = round256(mx_gemm_workspace_bytes(M, N, K, opts));
+    Item it = {};
+    it.index = i; it.ws_off = off; it.ws_bytes = b;
+    off += b;
+    if (A[i].ndim == 2 && B[i].ndim == 2 && (M == 0 || N == 0)) continue;   // empty problem
+    const int rc = gemm_impl(&A[i], &As[i], &B[i], &Bs[i], &C[i], opts, (uint8_t*)workspace + it.ws_off, it.ws_bytes,
+                             stream, &it.plan);
+    if (rc < 0) {
+      char inner[400];
+      snprintf(inner, sizeof inner, "%s", mx_last_error());
+      return set_error(rc, "problem %d of the list: %s", (int)i, inner);
+    }
+    it.simple = rc == MX_OK;
+    items.push_back(it);
+  }
+  // Pass 2: one scale re-layout launch per 64 scale tensors, one persistent GEMM launch per 32 problems of one
+  // element-format pair and output type
+  std::vector<PackArgs> packs;
+  for (const Item& it : items) {
+    if (!it.simple) continue;
+    if (it.plan.pack_a) packs.push_back(it.plan.pa);
+    if (it.plan.pack_b) packs.push_back(it.plan.pb);
+  }
+  if (!packs.empty())
+    if (int rc = launch_pack_scales_list(packs.data(), (int)packs.size(), (hipStream_t)stream)) return rc;
+  std::vector<char> done(items.size(), 0);
+  for (size_t i = 0; i < items.size(); ++i) {
+    if (!items[i].simple || done[i]) continue;
+    std::vector<GemmArgs> group;
+    const GemmArgs& g0 = items[i].plan.g;
+    for (size_t j = i; j < items.size(); ++j) {
+      const GemmArgs& g = items[j].plan.g;
+      if (items[j].simple && !done[j] && g.a_fmt == g0.a_fmt && g.b_fmt == g0.b_fmt && g.c_dtype == g0.c_dtype) {
+        group.push_back(g);
+        done[j] = 1;
+      }
+    }
+    if (int rc = launch_gemm_mfma_list(group.data(), (int)group.size(), (hipStream_t)stream)) return rc;
+  }
+  // Pass 3: the rest (large problems for the persistent 256 x 256 kernel, skinny ones for the decode kernel,
+  // split-K, batched operands, layouts only the general kernel reads), one call each
+  for (const Item& it : items) {
+    if (it.simple) continue;
+    const int32_t i = it.index;
+    const int rc = mx_gemm(&A[i], &As[i], &B[i], &Bs[i], &C[i], opts, (uint8_t*)workspace + it.ws_off, it.ws_bytes, stream);
     if (rc != MX_OK) {
       char inner[400];
       snprintf(inner, sizeof inner, "%s", mx_last_error());

@@ -379,12 +379,22 @@ __device__ inline int64_t scale_src_offset(const PackArgs& p, int64_t srow, int6
   return srow * p.s_row + kb * p.s_kb;
 }
 
-__global__ __launch_bounds__(256) void pack_scales_kernel(const PackPair pp) {
+// up to kPackListMax plain 2-D scale tensors (the operands of a list of problems) in one launch; the entries are
+// kept small so that the table travels as a kernel argument
+constexpr int kPackListMax = 64;
+struct PackEntry {
+  const uint8_t* src; uint32_t* dst;
+  int64_t rows, K, s_row, s_kb;
+};
+struct PackList {
+  PackEntry p[kPackListMax];
+  int32_t first_block[kPackListMax + 1];   // workgroups [first_block[i], first_block[i + 1]) belong to p[i]
+  int32_t n;
+};
+
+__device__ inline void pack_scales_block(const PackArgs& p, const int64_t blk) {
   constexpr int LD = 68;   // LDS row pitch (bytes): 64 scale bytes + 4 so that rows start on distinct banks
   __shared__ __attribute__((aligned(16))) uint8_t tile[64 * LD];
-  const bool second = (int)blockIdx.x >= pp.blocks0;
-  const PackArgs& p = second ? pp.p[1] : pp.p[0];
-  const int64_t blk = second ? blockIdx.x - pp.blocks0 : blockIdx.x;
   const int64_t KB = p.K / 32;
   const int64_t KQ = packed_scale_quads(p.K);
   const int64_t qgroups = (KQ + 3) / 4, rgroups = (p.rows + 63) / 64;
@@ -442,6 +452,21 @@ __global__ __launch_bounds__(256) void pack_scales_kernel(const PackPair pp) {
   }
   uint32_t* dst = p.dst + b * packed_scale_dwords(p.rows, p.K) + ((t64 * KQ + Q0 + q) * 64 + lane) * 4;
   *(uint4*)dst = make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+__global__ __launch_bounds__(256) void pack_scales_kernel(const PackPair pp) {
+  const bool second = (int)blockIdx.x >= pp.blocks0;
+  pack_scales_block(second ? pp.p[1] : pp.p[0], second ? blockIdx.x - pp.blocks0 : blockIdx.x);
+}
+
+__global__ __launch_bounds__(256) void pack_scales_list_kernel(const PackList pl) {
+  int i = 0;
+  while (i + 1 < pl.n && (int)blockIdx.x >= pl.first_block[i + 1]) ++i;   // uniform per workgroup
+  const PackEntry& e = pl.p[i];
+  PackArgs p = {};
+  p.src = e.src; p.dst = e.dst; p.rows = e.rows; p.K = e.K; p.s_row = e.s_row; p.s_kb = e.s_kb;
+  p.layout = MX_SCALE_2D; p.batch = 1; p.replicas = 1;
+  pack_scales_block(p, (int)blockIdx.x - pl.first_block[i]);
 }
 
 // ================================================================================================
@@ -681,6 +706,30 @@ int launch_pack_scales_pair(const PackArgs* a, const PackArgs* b, hipStream_t st
   hipLaunchKernelGGL(pack_scales_kernel, dim3((unsigned)total), dim3(256), 0, stream, pp);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "pack_scales_kernel launch: %s", hipGetErrorString(e));
+  return MX_OK;
+}
+
+int launch_pack_scales_list(const PackArgs* list, int n, hipStream_t stream) {
+  for (int i0 = 0; i0 < n; i0 += kPackListMax) {
+    PackList pl = {};
+    int64_t total = 0;
+    for (int i = i0; i < n && i < i0 + kPackListMax; ++i) {
+      const PackArgs& p = list[i];
+      if (p.rows <= 0 || p.K <= 0 || p.batch <= 0) continue;
+      if (p.layout != MX_SCALE_2D || p.batch != 1 || p.gather_ids)
+        return set_error(MX_ERR_INVALID, "pack_scales list: plain 2-D scale tensors only");
+      pl.p[pl.n] = PackEntry{p.src, p.dst, p.rows, p.K, p.s_row, p.s_kb};
+      pl.first_block[pl.n] = (int32_t)total;
+      total += ((p.rows + 63) / 64) * ((packed_scale_quads(p.K) + 3) / 4) * p.batch;
+      if (total > 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "pack_scales: tensors too large");
+      ++pl.n;
+    }
+    if (pl.n == 0) continue;
+    pl.first_block[pl.n] = (int32_t)total;
+    hipLaunchKernelGGL(pack_scales_list_kernel, dim3((unsigned)total), dim3(256), 0, stream, pl);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "pack_scales_list_kernel launch: %s", hipGetErrorString(e));
+  }
   return MX_OK;
 }
 

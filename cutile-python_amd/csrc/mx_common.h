@@ -103,6 +103,10 @@ struct GemmArgs {
 };
 
 int launch_gemm_mfma(const GemmArgs& g, int kernel_id, hipStream_t stream);
+// A list of independent plain products (no grouping, no split-K, one element format pair and output dtype for the
+// whole list) on the 128 x 128 one-tile kernel body: one persistent launch per 32 problems walks the concatenated
+// tile list (the scheme of grouped_matmul_kernel, test/kernels/group_gemm.py:10-38).
+int launch_gemm_mfma_list(const GemmArgs* problems, int n, hipStream_t stream);
 int launch_gemm_pingpong(const GemmArgs& g, hipStream_t stream);
 // the 32x32x64-instruction variant: 8-bit element formats only
 bool pingpong32_supports(int a_fmt, int b_fmt);
@@ -144,6 +148,8 @@ struct PackArgs {
 int launch_pack_scales(const PackArgs& p, hipStream_t stream);
 // both operands of one GEMM in a single launch; either pointer may be null
 int launch_pack_scales_pair(const PackArgs* a, const PackArgs* b, hipStream_t stream);
+// any number of plain 2-D scale tensors (64 per launch)
+int launch_pack_scales_list(const PackArgs* list, int n, hipStream_t stream);
 
 struct QuantArgs {
   const void* x; uint8_t* xq; uint8_t* scale;

@@ -32,11 +32,9 @@
 namespace mx {
 namespace {
 
+// One BM x BN tile of C: `pid` is the workgroup's number among the tiles of the problem, `split` its K slice.
 template <class C, typename OutT, bool GROUPED>
-__global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
-  lds_u8* const smem = (lds_u8*)smem_generic;
-
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, lds_u8* const smem, const int pid, const int split) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -48,7 +46,6 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
   int tile_m, tile_n, tile_lid;
   {
     const int total = tiles_m * tiles_n;
-    const int pid = blockIdx.x;
     // workgroup ids are dealt round-robin to the 8 XCDs (each has its own L2): give every XCD one
     // contiguous range of the logical tile order
     const int xcd = pid & 7, loc = pid >> 3, per = total >> 3, rem = total & 7;
@@ -67,7 +64,6 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
   // Split-K: blockIdx.y owns the K range [split * g.K, (split + 1) * g.K) of the full problem (g.K is the
   // slice length, a whole number of K-quads), its own slice of the packed scales and its own fp32 partial
   // output; a reduction kernel adds the partials.
-  const int split = blockIdx.y;
   const int ka0 = split * (g.K * C::A_EB / 8), kb0 = split * (g.K * C::B_EB / 8);   // first byte of the slice
   const int Kb_a = ka0 + g.K * C::A_EB / 8, Kb_b = kb0 + g.K * C::B_EB / 8;         // end of the slice in a row
   const int ksteps = (g.K + 127) / 128;
@@ -264,6 +260,66 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
 }
 
 template <class C, typename OutT, bool GROUPED>
+__global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
+  gemm_tile<C, OutT, GROUPED>(g, (lds_u8*)smem_generic, blockIdx.x, blockIdx.y);
+}
+
+// ---- list of problems: persistent workgroups walk the concatenated tile list -----------------------------------
+constexpr int kListMax = 32;
+struct ListProblem {
+  const uint8_t* A; const uint8_t* B; const uint32_t* As; const uint32_t* Bs; void* C;
+  int64_t lda, ldb, ldc;
+  int32_t M, N, K, accumulate;
+};
+struct GemmList {
+  ListProblem p[kListMax];
+  int32_t first_tile[kListMax + 1];
+  int32_t n, a_fmt, b_fmt, c_dtype;
+};
+
+template <class C, typename OutT>
+__global__ __launch_bounds__(C::NT) void gemm_list_kernel(const GemmList gl) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
+  const int total = gl.first_tile[gl.n];
+  for (int t = blockIdx.x; t < total; t += gridDim.x) {   // uniform per workgroup
+    int i = 0;
+    while (i + 1 < gl.n && t >= gl.first_tile[i + 1]) ++i;
+    const ListProblem& q = gl.p[i];
+    GemmArgs g = {};
+    g.A = q.A; g.B = q.B; g.As = q.As; g.Bs = q.Bs; g.C = q.C;
+    g.lda = q.lda; g.ldb = q.ldb; g.ldc = q.ldc;
+    g.M = q.M; g.N = q.N; g.K = q.K;
+    g.a_fmt = gl.a_fmt; g.b_fmt = gl.b_fmt; g.c_dtype = gl.c_dtype; g.accumulate = q.accumulate;
+    g.a_rows = q.M; g.replicas = 1;
+    gemm_tile<C, OutT, false>(g, (lds_u8*)smem_generic, t - gl.first_tile[i], 0);
+    // the tile's trailing (zero-fill) DMA has left the queue and every wave is done with the LDS stages before
+    // the next tile's loads reuse them
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+  }
+}
+
+template <class C, typename OutT>
+int launch_list_one(const GemmList& gl, hipStream_t stream) {
+  auto kern = gemm_list_kernel<C, OutT>;
+  static int attr_done = 0;   // benign race: the attribute call is idempotent
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if (e != hipSuccess)
+      return set_error(MX_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
+    attr_done = 1;
+  }
+  const int total = gl.first_tile[gl.n];
+  if (total <= 0) return MX_OK;
+  const int grid = total < 1024 ? total : 1024;   // 128 x 128 tiles: up to four workgroups per CU are resident
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::LDS_BYTES, stream, gl);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "gemm_list_kernel launch: %s", hipGetErrorString(e));
+  return MX_OK;
+}
+
+template <class C, typename OutT, bool GROUPED>
 int launch_one(const GemmArgs& g, hipStream_t stream) {
   auto kern = gemm_kernel<C, OutT, GROUPED>;
   static int attr_done = 0;   // benign race: the attribute call is idempotent
@@ -306,6 +362,43 @@ int launch_fmt(const GemmArgs& g, hipStream_t stream) {
 }
 
 }  // namespace
+
+int launch_gemm_mfma_list(const GemmArgs* problems, int n, hipStream_t stream) {
+  for (int i0 = 0; i0 < n; i0 += kListMax) {
+    GemmList gl = {};
+    int64_t total = 0;
+    for (int i = i0; i < n && i < i0 + kListMax; ++i) {
+      const GemmArgs& g = problems[i];
+      if (g.a_fmt != problems[0].a_fmt || g.b_fmt != problems[0].b_fmt || g.c_dtype != problems[0].c_dtype ||
+          g.sorted_token_ids || g.k_splits > 1)
+        return set_error(MX_ERR_INVALID, "gemm list: problems of one launch must share formats and be plain products");
+      ListProblem& q = gl.p[gl.n];
+      q.A = g.A; q.B = g.B; q.As = g.As; q.Bs = g.Bs; q.C = g.C;
+      q.lda = g.lda; q.ldb = g.ldb; q.ldc = g.ldc;
+      q.M = g.M; q.N = g.N; q.K = g.K; q.accumulate = g.accumulate;
+      gl.first_tile[gl.n] = (int32_t)total;
+      total += (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
+      if (total > 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "gemm list: too many tiles");
+      ++gl.n;
+    }
+    gl.first_tile[gl.n] = (int32_t)total;
+    gl.a_fmt = problems[0].a_fmt; gl.b_fmt = problems[0].b_fmt; gl.c_dtype = problems[0].c_dtype;
+    int rc = MX_ERR_DTYPE;
+#define MX_CASE(AFMT, BFMT)                                                                       \
+    if (gl.a_fmt == AFMT && gl.b_fmt == BFMT) {                                                     \
+      using C = Cfg<AFMT, BFMT, 128, 128, 2, 2>;                                                    \
+      rc = gl.c_dtype == MX_F32 ? launch_list_one<C, float>(gl, stream) : launch_list_one<C, uint16_t>(gl, stream); \
+    }
+    MX_CASE(MX_E4M3, MX_E4M3)
+    MX_CASE(MX_E5M2, MX_E5M2)
+    MX_CASE(MX_E2M1, MX_E2M1)
+    MX_CASE(MX_E4M3, MX_E2M1)
+#undef MX_CASE
+    if (rc == MX_ERR_DTYPE) return set_error(MX_ERR_DTYPE, "gemm list: unsupported element format pair (%d, %d)", gl.a_fmt, gl.b_fmt);
+    if (rc != MX_OK) return rc;
+  }
+  return MX_OK;
+}
 
 int launch_gemm_mfma(const GemmArgs& g, int kernel_id, hipStream_t stream) {
   if (g.c_dtype != MX_F32 && g.c_dtype != MX_BF16)

@@ -173,11 +173,16 @@ MX_API int mx_gemm_static(const mx_tensor* A, const mx_tensor* A_scale, const mx
 /*
  * A list of independent block-scaled products C[i] = A[i] x B[i] (problem sizes may all differ), the
  * block-scaled counterpart of grouped_matmul_kernel(As, Bs, Cs, ...), test/kernels/group_gemm.py:10-38.
- * The descriptor arrays hold `count` entries each; every problem follows the rules of mx_gemm and is
- * enqueued on `stream` in list order (no host synchronisation; one workspace of
- * mx_gemm_list_workspace_bytes, the largest single need, is reused from problem to problem, which stream
- * order makes safe).  Empty problems (M or N zero) are skipped.  On error the index of the failing
- * problem is part of mx_last_error() and nothing after it is enqueued.
+ * The descriptor arrays hold `count` entries each; every problem follows the rules of mx_gemm.  All problems are
+ * validated first: on error the index of the failing problem is part of mx_last_error() and nothing has been
+ * enqueued.  Problems that mx_gemm would give to its 128 x 128 one-tile kernel (the small and medium ones, which
+ * is what such lists hold) run the way the reference's kernel does: one launch re-lays up to 64 scale
+ * tensors, and one launch of persistent workgroups walks the concatenated tile list of up to 32 problems of one
+ * element-format pair and output type (tile_idx += number of workgroups).  The others (large problems for the
+ * persistent 256 x 256 kernel, skinny ones for the decode kernel, split-K, layouts of the general kernel) get a
+ * call of their own behind them.  No host synchronisation.  The workspace holds one slice per problem
+ * (mx_gemm_list_workspace_bytes is the sum of the single needs): the problems run side by side.  Empty problems
+ * (M or N zero) are skipped.
  */
 MX_API int64_t mx_gemm_list_workspace_bytes(int32_t count, const mx_tensor* A, const mx_tensor* B,
                                      const mx_gemm_opts* opts);

@@ -205,6 +205,30 @@ def test_list_of_problems(ct, dev, kernel):
             _check(c, oracle_matmul(a, b), torch.float32, f"list {m}x{n}x{k}")
 
 
+def test_list_of_many_small_problems_matches_single_calls(ct, dev):
+    """test/test_group_gemm.py:14-34 drives grouped_matmul_kernel with lists of small problems, tiles larger than
+    a problem included.  70 problems (more than one persistent launch takes), ragged sizes from one tile row to a
+    few tiles, two element formats interleaved, one problem large enough to leave the batched path: every
+    result is bit-identical to the same problem run alone, and within tolerance of the oracle."""
+    rng = np.random.default_rng(5)
+    As, Ass, Bs, Bss, single = [], [], [], [], []
+    ops = []
+    for i in range(70):
+        m, n, k = int(rng.integers(1, 300)), int(rng.integers(1, 300)), 32 * int(rng.integers(1, 20))
+        if i == 40:
+            m, n, k = 3072, 3072, 512      # 144 tiles of 256 x 256: goes to the persistent 256 x 256 kernel
+        fmt = O.E4M3 if i % 3 else O.E5M2
+        a, b = randn_operand(m, k, fmt, 2000 + i, dev), randn_operand(n, k, fmt, 3000 + i, dev)
+        ops.append((a, b))
+        As.append(a.storage); Ass.append(a.scale_t); Bs.append(b.storage.T); Bss.append(b.scale_t.T)
+        single.append(_run(ct, a, b))
+    got = ct.grouped_block_scaled_matmul(As, Ass, Bs, Bss)
+    for i, ((a, b), c, c1) in enumerate(zip(ops, got, single)):
+        assert torch.equal(c, c1), i
+        if i % 10 == 0:
+            _check(c, oracle_matmul(a, b), torch.float32, f"list problem {i}")
+
+
 def test_list_of_problems_reports_the_failing_index(ct, dev):
     a = randn_operand(64, 64, O.E4M3, 1, dev)
     b = randn_operand(64, 64, O.E4M3, 2, dev)
