@@ -269,12 +269,22 @@ struct Decode2Cfg {
   static constexpr int WIW = 16 / RPI / 2;        // weight DMA instructions per wave and tile
   static constexpr int SROW = SPW * 16;           // scale bytes per weight row (K / 32)
   static constexpr int LS = SROW / 16;            // lanes per scale row
+  // XOR term of a scale row's 16-byte pieces in LDS: rows that start in the same bank differ in it
+  __device__ static constexpr int sswz(int row) { return (row * SROW / 256) % LS; }
   static constexpr int S_INSTR = 16 * SROW / 1024;   // scale DMA instructions per tile (waves 0 .. S_INSTR-1)
   static constexpr int W_BYTES = 4 * 16 * SLB;
   static constexpr int SLOT = W_BYTES + 16 * SROW;
   static constexpr int RING = 2 * SLOT;
   static constexpr int RED = kWaves * 64 * 16;       // partial sums of one tile: [wave][lane] float4
-  static constexpr int LDS_BYTES = RING + 2 * RED;   // two reduction buffers behind the ring
+  // Staging of X before the stream starts: XNB round buffers of 4 KiB per wave (16 rows x 256 bytes).  Tile 0 is in
+  // flight to slot 1 meanwhile, so the buffers sit inside slot 0 if that is large enough, else behind the reduction
+  // buffers; the X scales (1 KiB per wave) use the reduction buffers, which are idle until tile 0 is done.
+  static constexpr int XNB = 2;
+  static constexpr int XSTAGE = kWaves * XNB * 4096;
+  static constexpr int XSTAGE_OFF = XSTAGE <= SLOT ? 0 : RING + 2 * RED;
+  static constexpr int XSCALE_OFF = RING;
+  static constexpr int LDS_BYTES = XSTAGE <= SLOT ? RING + 2 * RED : RING + 2 * RED + XSTAGE;
+  static_assert(kWaves * 1024 <= 2 * RED, "X scale staging");
 };
 
 // The weight and scale DMA of one wave for one tile.  Instruction j of the wave covers rows
@@ -297,6 +307,20 @@ __device__ inline void issue_tile_dma2(const uint8_t* W, uint32_t wbytes, const 
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsS, (lds_void*)sdst, 16, soff, ssoff, 0, 0);
 }
 
+// The 4 LDS-DMA loads of one staging round of a wave: 256 bytes of each of 16 consecutive rows of X (4 rows per
+// instruction), row rr to dst + rr * 256
+__device__ inline void issue_x_round(const uint8_t* X, uint32_t xbytes, lds_u8* dst, const uint32_t* voff, int soff0,
+                                     int ldx) {
+  const __amdgpu_buffer_rsrc_t rsX = make_rsrc(X, xbytes);
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsX, (lds_void*)(dst + j * 1024), 16, voff[j], soff0 + 4 * j * ldx, 0, 0);
+}
+__device__ inline void issue_xs_dma(const uint8_t* Xs, uint32_t bytes, lds_u8* dst, uint32_t voff, int soff) {
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(Xs, bytes);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)dst, 16, voff, soff, 0, 0);
+}
+
 template <int XF, int SPW, typename OutT>
 __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d) {
   using Cf = Decode2Cfg<SPW>;
@@ -313,54 +337,91 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
   const int rl = lane / Cf::LPR;                 // row of the lane inside one DMA instruction
   const uint32_t row_off = (uint32_t)(rl * d.ldw);
   const uint32_t chunk_off = (uint32_t)((((lane % Cf::LPR) ^ rl) << 4) + q * Cf::SLB);   // SLB: no bits below 512
-  const uint32_t soff = (uint32_t)((wave * (64 / Cf::LS) + lane / Cf::LS) * d.ldws + (lane % Cf::LS) * 16);
-  auto issue = [&](int tile, int slot) {
+  // a scale row is SROW = 256 (128) bytes in LDS, so every (second) row starts in the same bank: the 16-byte
+  // pieces of a row are XOR-swizzled by the row like the weight chunks, and the 16 rows a fragment read touches
+  // sit in 16 different bank groups
+  const int srow = wave * (64 / Cf::LS) + lane / Cf::LS;
+  const uint32_t soff = (uint32_t)(srow * d.ldws + (((lane % Cf::LS) ^ Cf::sswz(srow)) * 16));
+  // Tiles of this workgroup: local tile i is tile t_first + i G (16 consecutive weight rows), so that the workgroups
+  // together read one contiguous window of G tiles at a time.  Workgroup ids go round-robin over the 8 XCDs; XCD x
+  // takes the x-th eighth of every window, so that every XCD reads from all address slices instead of always the
+  // same eighth of them (measured 1.1 us of 29 at the 28672 x 8192 weights; two windows of 8-row half tiles, which
+  // a pure streaming test prefers, measure 2 us slower here).
+  const int tiles = d.N / 16;
+  const int G = gridDim.x;
+  const int t_first = G % 8 == 0 ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x;
+  const int t_count = t_first < tiles ? (tiles - t_first + G - 1) / G : 0;
+  auto issue = [&](int i, int slot) {          // this wave's share of local tile i
+    const int tile = t_first + i * G;
     lds_u8* const base = smem + slot * Cf::SLOT;
     issue_tile_dma2<SPW>(d.W, wbytes, d.Ws, sbytes, base + q * (16 * Cf::SLB) + mh * Cf::WIW * 1024,
                          base + Cf::W_BYTES + wave * 1024, row_off, chunk_off, mh * Cf::WIW * Cf::RPI, soff,
                          tile * 16 * (int)d.ldw, (int)d.ldw, tile * 16 * (int)d.ldws, with_scales);
   };
 
-  // tiles of this workgroup: blockIdx.x, + gridDim.x, ... -- at any moment the workgroups together read one
-  // contiguous window of W (gridDim.x tiles of 16 rows), which spreads evenly over the memory channels
-  const int tiles = d.N / 16;
-  const int G = gridDim.x, t_first = blockIdx.x;
-  const int t_count = t_first < tiles ? (tiles - t_first + G - 1) / G : 0;
   if (t_count == 0) return;                    // uniform per workgroup
 
-  // ---- resident X: rows 16 mh + r, K-steps q SPW .. of it, requested before the W stream ----------------
-  // Buffer loads: rows at or beyond M are out of range and read as zeros (elements 0, scale byte 0 = 2^-127),
-  // so the operand registers are written by the loads themselves, with no masking pass over them.
+  // ---- resident X: rows 16 mh + r, K-steps q SPW .. of it ------------------------------------------------------
+  // X comes through LDS: a DMA instruction reads 256 contiguous bytes of each of 4 rows of X, and the wave then picks
+  // its operand registers out of its own staging area.  (Loading the operand layout straight from memory, 16 rows
+  // x 64 bytes per instruction and every workgroup the same 264 KiB, keeps the texture-address unit and L2 busy for
+  // 6 us at the 32 x 8192 activations; this way the 256 KiB cross the CU's 64-byte/clock memory port in 3 us.)  A round
+  // is two K-steps: 16 rows x 256 bytes per wave, 16-byte chunks XOR-swizzled by row; two rounds are in flight.  Rows
+  // at or beyond M are out of range of the descriptor and arrive as zeros (scale byte 0 = 2^-127).
+  // The DMA of tile 0 is requested first: the memory pipe returns data in request order for the whole CU, so X
+  // arrives behind it, but HBM has something to do meanwhile (0.7 us faster than staging X first); with both first
+  // tiles in flight there would be no room in LDS to stage X.
   v8i xf[SPW];
   int xs[SPW / 4];
   {
-    const __amdgpu_buffer_rsrc_t rsX = make_rsrc(d.X, (uint32_t)((int64_t)d.M * d.ldx));
-    const __amdgpu_buffer_rsrc_t rsXs = make_rsrc(d.Xs, (uint32_t)((int64_t)d.M * d.ldxs));
-    const int m = 16 * mh + r;
-    const uint32_t xoff = (uint32_t)(m * d.ldx + q * SPW * 128 + gq * 16);
-    const uint32_t xsoff = (uint32_t)(m * d.ldxs + q * SPW * 4);
-    v4i xsraw[SPW / 4];
+    constexpr int XR = SPW / 2;                       // rounds
+    issue(0, 1);                                       // tile i lives in slot (i + 1) % 2
+    lds_u8* const xst = smem + Cf::XSTAGE_OFF + wave * (Cf::XNB * 4096);
+    lds_u8* const xsst = smem + Cf::XSCALE_OFF + wave * 1024;
+    const uint32_t xbytes = (uint32_t)((int64_t)d.M * d.ldx);
+    uint32_t xvo[4];                                  // lane offsets of the 4 DMA instructions of a round
 #pragma unroll
-    for (int s = 0; s < SPW; ++s) {
-      const v4i lo = __builtin_amdgcn_raw_buffer_load_b128(rsX, xoff, s * 128, 0);
-      const v4i hi = __builtin_amdgcn_raw_buffer_load_b128(rsX, xoff, s * 128 + 64, 0);
-      xf[s] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    for (int j = 0; j < 4; ++j) xvo[j] = (uint32_t)((lane >> 4) * d.ldx + (((lane & 15) ^ (4 * j + (lane >> 4))) << 4));
+    const int xso = 16 * mh * (int)d.ldx + q * SPW * 128;
+    // the wave's own X scales: 16 rows x SPW * 4 bytes, one instruction
+    {
+      constexpr int LPRS = SPW * 4 / 16;              // lanes per row
+      const int srw = lane / LPRS;
+      issue_xs_dma(d.Xs, (uint32_t)((int64_t)d.M * d.ldxs), xsst,
+                   srw < 16 ? (uint32_t)(srw * d.ldxs + (lane % LPRS) * 16) : kOob, 16 * mh * (int)d.ldxs + q * SPW * 4);
     }
 #pragma unroll
-    for (int u = 0; u < SPW / 4; ++u) {
-      xsraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rsXs, xsoff, u * 16, 0);
+    for (int h = 0; h < Cf::XNB && h < XR; ++h) issue_x_round(d.X, xbytes, xst + h * 4096, xvo, xso + h * 256, (int)d.ldx);
+#pragma unroll
+    for (int h = 0; h < XR; ++h) {
+      static_assert(Cf::XNB == 2, "wait counts below");
+      if (h + 1 < XR) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);   // round h + 1 may stay in flight
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
+      asm volatile("" ::: "memory");
+      lds_u8* const row = xst + (h % Cf::XNB) * 4096 + r * 256;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const v4i lo = *(lds_cv4i*)(row + (((s2 * 8 + gq) ^ r) << 4));
+        const v4i hi = *(lds_cv4i*)(row + (((s2 * 8 + 4 + gq) ^ r) << 4));
+        xf[h * 2 + s2] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+      if (h == 0) {                                    // the scales landed before round 0
+#pragma unroll
+        for (int u = 0; u < SPW / 4; ++u) {
+          const v4i raw = *(lds_cv4i*)(xsst + r * (SPW * 4) + u * 16);
+          uint32_t pk = 0;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) pk |= (((uint32_t)raw[t] >> (8 * gq)) & 0xFFu) << (8 * t);
+          xs[u] = (int)pk;
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // round h + XNB (or the weight stream) overwrites the buffer
+      if (h + Cf::XNB < XR)
+        issue_x_round(d.X, xbytes, xst + (h % Cf::XNB) * 4096, xvo, xso + (h + Cf::XNB) * 256, (int)d.ldx);
     }
+    __syncthreads();                                   // the weight slots overlap the other waves' staging areas
+    if (t_count > 1) issue(1, 0);
     __builtin_amdgcn_sched_barrier(0);
-    issue(t_first, 0);
-    if (t_count > 1) issue(t_first + G, 1);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int u = 0; u < SPW / 4; ++u) {
-      uint32_t pk = 0;
-#pragma unroll
-      for (int t = 0; t < 4; ++t) pk |= (((uint32_t)xsraw[u][t] >> (8 * gq)) & 0xFFu) << (8 * t);
-      xs[u] = (int)pk;
-    }
   }
 
   // ---- per tile: partial sums of the 4 K-slices meet in LDS and leave while the next tiles stream in -------
@@ -419,14 +480,14 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
     // multiplications start.  The scales first, packed to the lane's own byte of each K-step (one register
     // per four K-steps): with the 16 raw scale registers alive next to the fragments the kernel would spill,
     // and a spill reload queues behind the DMA just issued.
-    lds_u8* const wt = smem + (i & 1) * Cf::SLOT + q * (16 * Cf::SLB) + r * Cf::SLB;
-    lds_u8* const st = smem + (i & 1) * Cf::SLOT + Cf::W_BYTES + r * Cf::SROW + q * (SPW * 4);
+    lds_u8* const wt = smem + ((i + 1) & 1) * Cf::SLOT + q * (16 * Cf::SLB) + r * Cf::SLB;
+    lds_u8* const st = smem + ((i + 1) & 1) * Cf::SLOT + Cf::W_BYTES + r * Cf::SROW;
     int ws[SPW / 4];
     v4i w[SPW];
     {
 #pragma unroll
       for (int h = 0; h < SPW / 4; ++h) {
-        const v4i sc = *(lds_cv4i*)(st + 16 * h);
+        const v4i sc = *(lds_cv4i*)(st + (((q * (SPW / 4) + h) ^ Cf::sswz(r)) << 4));
         uint32_t pk = 0;
 #pragma unroll
         for (int t = 0; t < 4; ++t) pk |= (((uint32_t)sc[t] >> (8 * gq)) & 0xFFu) << (8 * t);
@@ -444,7 +505,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    if (i + 2 < t_count) issue(t_first + (i + 2) * G, i & 1);
+    if (i + 2 < t_count) issue(i + 2, (i + 1) & 1);
     __builtin_amdgcn_sched_barrier(0);
     if (i > 0 && wave < 2) reduce_store(i - 1);   // uniform per wave
     v4f acc[2] = {(v4f){0.f, 0.f, 0.f, 0.f}, (v4f){0.f, 0.f, 0.f, 0.f}};   // even / odd K-steps: two MFMA chains
@@ -528,6 +589,7 @@ int launch_decode_x(const DecodeArgs& d, int grid, hipStream_t stream) {
 }
 
 }  // namespace
+
 
 int launch_gemm_decode(const DecodeArgs& d, hipStream_t stream) {
   if (d.w_fmt != MX_E2M1) return set_error(MX_ERR_DTYPE, "decode kernel: weights must be MX_E2M1");
