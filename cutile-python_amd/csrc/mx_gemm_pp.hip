@@ -106,10 +106,24 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     for (int j = 0; j < 4; ++j) sb[j] = Bs1[(int64_t)idx16 * 4 + 16 * (j & 1) + 2 * (j >> 1)];
   };
   bool fetch_valid = true;   // false once the walk has no further tile: loads become zero-fill no-ops
+  // grouped: this team's 128 rows of the tile are all alignment padding (the padding of an expert's block is its
+  // tail, and blocks are whole tiles, so it is enough to look at the first row of the half).  Such a half has
+  // nothing to multiply: its fragment reads and MFMAs are skipped, which is what makes a half-filled tile cost
+  // about as much as a 128-row tile would.
+  bool skip_cur = false, skip_nxt = false;
   auto set_fetch_tile = [&](int lid) {
     fetch_valid = lid < walk.end;
     int m0 = 0, n0 = 0;
     if (fetch_valid) walk.origin(lid, m0, n0);
+    if constexpr (GROUPED) {
+      skip_nxt = false;
+      if (fetch_valid && m0 + wm0 < g.M) {
+        const int id0 = g.sorted_token_ids[m0 + wm0];
+        skip_nxt = id0 < 0 || id0 >= g.num_valid_ids;
+      } else if (fetch_valid) {
+        skip_nxt = true;
+      }
+    }
     int expert = 0;
     if constexpr (GROUPED) expert = g.sorted_expert_ids[m0 / g.tile_m];
     const uint8_t* Bbase = g.B + (GROUPED ? (int64_t)expert * g.b_expert_stride : 0);
@@ -320,12 +334,14 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     lds_u8* const btile = smem + P::B_BASE + bbuf * C::B_STAGE + (wn0 + bperm_lane_off(r)) * C::B_RB;
     issue_a(sl_eff, abuf2);
     v8i bf[C::KSUB][4], af[C::KSUB][8];
+    if (!(GROUPED && skip_cur)) {
 #pragma unroll
-    for (int kk = 0; kk < C::KSUB; ++kk) {
+      for (int kk = 0; kk < C::KSUB; ++kk) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) bf[kk][j] = load_frag<C::B_RB, C::B_EB>(btile, bperm_tile_off(j), kk, gq, swb);
+        for (int j = 0; j < 4; ++j) bf[kk][j] = load_frag<C::B_RB, C::B_EB>(btile, bperm_tile_off(j), kk, gq, swb);
 #pragma unroll
-      for (int i = 0; i < EARLY; ++i) af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
+        for (int i = 0; i < EARLY; ++i) af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
+      }
     }
     if constexpr (TEAM == 1) {
       // the B buffer of this stage is free once this wave's own reads have returned
@@ -372,10 +388,12 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       __builtin_amdgcn_sched_barrier(0);
     };
     // A tiles below EARLY were read in the memory phase; the rest is read EARLY * 4 MFMAs ahead of use
+    if (!(GROUPED && skip_cur)) {
 #pragma unroll
-    for (int ip = 0; ip < 8; ip += 2) {
-      if (ip + EARLY < 8) read_pair(ip + EARLY);
-      mfma_pair(ip);
+      for (int ip = 0; ip < 8; ip += 2) {
+        if (ip + EARLY < 8) read_pair(ip + EARLY);
+        mfma_pair(ip);
+      }
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
@@ -390,6 +408,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     bbuf ^= 1;
   };
   for (; lid < walk.end; lid += walk.step) {
+    skip_cur = skip_nxt;
     as_cur[0] = as_nxt[0];
     as_cur[1] = as_nxt[1];
     bs_cur = bs_nxt;

@@ -10,7 +10,7 @@ include/mxgemm.h; see ops.py for the reference counterparts of each function.
 """
 from ._lib import LIB_PATH, MXLibraryError, lib
 from .errors import TileTypeError, TileValueError
-from .ops import (PackedScales, bench_block_scaled_matmul, block_quantize, block_scaled_matmul, cutile_block_scaled_matmul,
+from .ops import (PackedScales, bench_block_scaled_matmul, block_quantize, clear_scale_cache, block_scaled_matmul, cutile_block_scaled_matmul,
                   cutile_moe_scaled, grouped_block_scaled_matmul, invoke_fused_moe_scaled, mma_scaled, moe_align_tile_size, pack_scales,
                   silu_and_mul_quantize, swizzle_32_4_4, unswizzle_32_4_4)
 
@@ -19,4 +19,5 @@ __all__ = [
     "block_quantize", "block_scaled_matmul", "cutile_block_scaled_matmul", "invoke_fused_moe_scaled",
     "mma_scaled", "moe_align_tile_size", "pack_scales", "swizzle_32_4_4", "unswizzle_32_4_4",
     "silu_and_mul_quantize", "cutile_moe_scaled", "grouped_block_scaled_matmul", "bench_block_scaled_matmul",
+    "clear_scale_cache",
 ]

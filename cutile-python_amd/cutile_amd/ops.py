@@ -17,8 +17,10 @@ Reference counterparts
 """
 from __future__ import annotations
 
+import collections
 import ctypes
 import threading
+import weakref
 from dataclasses import dataclass
 from typing import Optional, Tuple
 
@@ -145,6 +147,57 @@ def _scale_desc(s, rows: int, K: int, block: int, is_b: bool):
     return L.desc(_as_u8(s), code), L.MX_SCALE_2D
 
 
+class _ScaleCache:
+    """PackedScales of scale tensors that were passed before (``cache_scales=True``): what the reference gets by
+    reading swizzle_32_4_4 scales in place (test/kernels/scaled_matmul.py:77-104), a weight's scales cost one
+    re-layout here instead of one per call.  An entry belongs to a tensor OBJECT (the base tensor of a view, held
+    by weak reference) at one ``_version``: a new tensor at the same address, a tensor that died, or one that torch
+    has written to since never match.  Writes that bypass torch's version counter (another library writing through
+    the raw pointer) are not seen; callers that do that must not ask for caching."""
+
+    def __init__(self, max_entries: int = 64):
+        self.max_entries = max_entries
+        self._lock = threading.Lock()
+        self._entries = collections.OrderedDict()   # key -> (weakref to base, version, PackedScales, event, stream)
+
+    def clear(self):
+        with self._lock:
+            self._entries.clear()
+
+    def lookup(self, s: torch.Tensor, transposed: bool) -> PackedScales:
+        base = s._base if s._base is not None else s
+        key = (id(base), s.data_ptr(), tuple(s.shape), tuple(s.stride()), s.dtype, transposed)
+        stream = torch.cuda.current_stream(s.device)
+        with self._lock:
+            e = self._entries.get(key)
+            if e is not None and e[0]() is base and e[1] == base._version:
+                self._entries.move_to_end(key)
+                if e[4] != stream.cuda_stream:
+                    stream.wait_event(e[3])          # the re-layout ran on another stream
+                return e[2]
+        packed = pack_scales(s, transposed=transposed)
+        if torch.cuda.is_current_stream_capturing():
+            return packed                             # memory of the capture's private pool: not for later eager calls
+        ev = torch.cuda.Event()
+        ev.record(stream)
+        with self._lock:
+            self._entries[key] = (weakref.ref(base), base._version, packed, ev, stream.cuda_stream)
+            # entries of dead tensors first, then the least recently used
+            for k in [k for k, v in self._entries.items() if v[0]() is None]:
+                del self._entries[k]
+            while len(self._entries) > self.max_entries:
+                self._entries.popitem(last=False)
+        return packed
+
+
+_SCALE_CACHE = _ScaleCache()
+
+
+def clear_scale_cache() -> None:
+    """Drops every cached scale re-layout (see ``cache_scales`` of :func:`block_scaled_matmul`)."""
+    _SCALE_CACHE.clear()
+
+
 _WS_LOCAL = threading.local()
 
 
@@ -181,8 +234,24 @@ def _gemm_descs(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, block):
     return (dA, dAs, dB, dBs, dC), (la, lb), (M, N, K)
 
 
+def _cacheable_scale(s, block: int) -> bool:
+    return (isinstance(s, torch.Tensor) and block == 32 and s.dim() in (2, 4) and _scale_code(s) == L.MX_E8M0)
+
+
 def _launch_gemm(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, *, accumulate, kernel, block, split_k=0,
-                 static_scratch=False):
+                 static_scratch=False, cache_scales=False):
+    if cache_scales and kernel != "generic" and A.dim() == 2 and B.dim() == 2 and \
+            (_cacheable_scale(As, block) or _cacheable_scale(Bs, block)):
+        # Native-layout scales are only read by the MFMA kernels: a problem that needs the general kernel reports
+        # that before anything is enqueued, and runs with the scales as given.
+        As_c = _SCALE_CACHE.lookup(As, False) if _cacheable_scale(As, block) else As
+        Bs_c = _SCALE_CACHE.lookup(Bs, True) if _cacheable_scale(Bs, block) else Bs
+        try:
+            return _launch_gemm(A, a_fmt, a_pd, As_c, B, b_fmt, b_pd, Bs_c, C, accumulate=accumulate, kernel=kernel,
+                                block=block, split_k=split_k, static_scratch=static_scratch)
+        except (RuntimeError, ValueError, TypeError) as e:
+            if "native-layout" not in str(e):
+                raise
     dev = A.device
     (dA, dAs, dB, dBs, dC), (la, lb), (M, N, K) = _gemm_descs(A, a_fmt, a_pd, As, B, b_fmt, b_pd, Bs, C, block)
     o = _opts(accumulate, la, lb, kernel, block, split_k)
@@ -259,7 +328,7 @@ def block_scaled_matmul(A: torch.Tensor, A_scale, B: torch.Tensor, B_scale, *,
                         out_dtype: torch.dtype = torch.float32, C: Optional[torch.Tensor] = None,
                         accumulate: bool = False, a_format: Optional[str] = None,
                         b_format: Optional[str] = None, kernel: str = "auto", split_k: int = 0,
-                        static_scratch: bool = False) -> torch.Tensor:
+                        static_scratch: bool = False, cache_scales: bool = False) -> torch.Tensor:
     """C = (A * A_scale) @ (B * B_scale) with fp32 accumulation, returned as ``out_dtype``.
 
     A (M, K) and B (K, N) hold MX elements: ``float8_e4m3fn`` / ``float8_e5m2``, or FP4 E2M1 packed two
@@ -275,6 +344,9 @@ def block_scaled_matmul(A: torch.Tensor, A_scale, B: torch.Tensor, B_scale, *,
     (``mx_gemm_static``) instead of a torch allocation; with a preallocated ``C`` the call then allocates
     nothing.  Problems that need more than ``lib().mx_static_scratch_bytes()`` raise ``ValueError``; calls that
     overlap on one GPU (several streams or threads) must not share it.
+    ``cache_scales``: keep the MFMA-ready re-layout of every 2-D / swizzle_32_4_4 scale tensor passed here and reuse
+    it while that tensor object lives and torch has not written to it (``_version``), so that repeated calls with
+    the same weights launch the GEMM kernel only; :func:`clear_scale_cache` drops the copies.
     """
     a_fmt, b_fmt = _elem_format(A, a_format), _elem_format(B, b_format)
     if a_fmt is None or b_fmt is None:
@@ -311,7 +383,8 @@ def block_scaled_matmul(A: torch.Tensor, A_scale, B: torch.Tensor, B_scale, *,
         if tuple(C.shape) != (m, n) or C.dtype not in (torch.float32, torch.bfloat16) or C.device != A.device:
             raise ValueError(f"C must be a ({m}, {n}) float32 or bfloat16 tensor on {A.device}")
     return _launch_gemm(A, a_fmt, a_pd, A_scale, B, b_fmt, b_pd, B_scale, C, accumulate=accumulate,
-                        kernel=kernel, block=32, split_k=split_k, static_scratch=static_scratch)
+                        kernel=kernel, block=32, split_k=split_k, static_scratch=static_scratch,
+                        cache_scales=cache_scales)
 
 
 def grouped_block_scaled_matmul(As, A_scales, Bs, B_scales, *, out_dtype: torch.dtype = torch.float32,

@@ -290,3 +290,43 @@ def test_four_wave_kernel_rejects_what_it_cannot_run(ct, dev):
     a4, b4 = randn_operand(256, 512, O.E2M1, 1, dev), randn_operand(256, 512, O.E2M1, 2, dev)
     with pytest.raises(ct.TileTypeError, match="8-bit"):
         _run(ct, a4, b4, kernel="w4p")
+
+
+def test_cached_scale_relayout(ct, dev):
+    """cache_scales=True: same bits as without, one re-layout per live scale tensor, recomputed after torch writes
+    to the tensor, and no effect on problems the general kernel runs."""
+    from cutile_amd import ops
+    ct.clear_scale_cache()
+    a = randn_operand(256, 512, O.E4M3, 71, dev)
+    b = randn_operand(384, 512, O.E4M3, 72, dev)
+    bs_t = b.scale_t.T                      # the view the sample passes; a new view object per call below
+    plain = ct.block_scaled_matmul(a.storage, a.scale_t, b.storage.T, bs_t)
+    c1 = ct.block_scaled_matmul(a.storage, a.scale_t, b.storage.T, b.scale_t.T, cache_scales=True)
+    assert len(ops._SCALE_CACHE._entries) == 2
+    c2 = ct.block_scaled_matmul(a.storage, a.scale_t, b.storage.T, b.scale_t.T, cache_scales=True)
+    assert len(ops._SCALE_CACHE._entries) == 2, "second call must hit both entries"
+    assert torch.equal(plain, c1) and torch.equal(plain, c2)
+    # swizzle_32_4_4 input
+    a_sw = ct.swizzle_32_4_4(a.scale_t)
+    c3 = ct.block_scaled_matmul(a.storage, a_sw, b.storage.T, b.scale_t.T, cache_scales=True)
+    assert torch.equal(plain, c3)
+    # torch writes to the scales: the stale copy must not be used
+    a.scale_t.view(torch.uint8).add_(1)     # every A scale doubled
+    c4 = ct.block_scaled_matmul(a.storage, a.scale_t, b.storage.T, b.scale_t.T, cache_scales=True)
+    assert torch.equal(c4, plain * 2)
+    # another stream uses the cached copy behind the event of the re-layout
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        c5 = ct.block_scaled_matmul(a.storage, a.scale_t, b.storage.T, b.scale_t.T, cache_scales=True)
+    s.synchronize()
+    assert torch.equal(c5, c4)
+    # a problem of the general kernel (row-major B) ignores the cache
+    b_rm = b.storage.T.contiguous()
+    ref = ct.block_scaled_matmul(a.storage, a.scale_t, b_rm, b.scale_t.T)
+    c6 = ct.block_scaled_matmul(a.storage, a.scale_t, b_rm, b.scale_t.T, cache_scales=True)
+    assert torch.equal(ref, c6)
+    # a dead tensor's entry never matches a new tensor at the same address
+    n_before = len(ops._SCALE_CACHE._entries)
+    del a_sw
+    ct.clear_scale_cache()
+    assert len(ops._SCALE_CACHE._entries) == 0 and n_before >= 2
