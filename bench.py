@@ -507,7 +507,7 @@ def main():
         extra["c3_decode_m32"] = {"gbs_wall_clock": r["gbs_wall"], "ms_per_step": r["ms_per_step"],
                                   "rel_fro_vs_oracle": r["rel_fro_vs_oracle"],
                                   "roofline": roofline("hbm", r["gbs"], PEAK_HBM_GBS, "GB/s", "c3",
-                                                       "decode2_kernel<e4m3,16,bf16>", r["kernel"], r["bytes"])}
+                                                       "decode_kernel<e4m3,16,bf16>", r["kernel"], r["bytes"])}
         torch.cuda.empty_cache()
     if "c5" in want:
         r = bench_moe(ct, O, dev, a.steps, a.warmup, check, full_forward=not a.no_moe_forward)

@@ -1,21 +1,24 @@
 // Skinny-M ("decode") block-scaled GEMM: C[M<=32, N] = X[M, K] (8-bit MX) x W[N, K] (MXFP4) ^T.
 //
-// The problem is bound by streaming W (and its scales) from HBM exactly once, so the kernel is
-// organised around long contiguous reads and many bytes in flight, not around tile reuse:
-//   * a workgroup of 8 waves takes every gridDim.x-th 16-row tile of W (64 KiB each at K = 8192);
-//     wave w owns K-slice w (SPW MFMA K-steps of 128 elements) of every tile, so the 8 waves together
-//     read a tile as one contiguous piece and the workgroups together one contiguous window of W;
-//   * W and its E8M0 scales go global -> LDS with buffer_load ... lds (no VGPR staging): two tiles per
-//     wave are in flight (144 KiB per CU) while the previous one is multiplied.  A wave only ever reads
-//     back what it loaded itself, so the streaming loop has no workgroup barrier, only s_waitcnt vmcnt;
-//   * each wave keeps its K-slice of X (and of the X scales) resident in VGPRs for the whole kernel (X is
-//     tiny and shared by all workgroups through L2), in the 8-bit MFMA operand layout: bytes
-//     16 g .. 16 g + 15 and 64 + 16 g .. of each K-step for lane group g;
-//   * v_mfma_scale_f32_16x16x128_f8f6f4 with mixed formats (W as FP4 first matrix, X as FP8 second
-//     matrix); W fragments are read from LDS (16-byte chunks XOR-swizzled by row: conflict free), the
-//     scale byte of the lane's block is shifted down to where op_sel 0 reads it;
-//   * partial sums of up to 8 tiles stay in registers; one LDS reduction over the 8 K-slices per batch
-//     of tiles, then 512 threads write the bf16/fp32 result.
+// The problem is bound by streaming W (and its scales) from HBM exactly once, so the kernel is organised around
+// long contiguous reads and many bytes in flight, not around tile reuse:
+//   * a workgroup of 8 waves takes every gridDim.x-th 16-row tile of W (64 KiB at K = 8192); the waves are
+//     4 K-slices x 2 halves of M (16 rows of X each): wave (q, mh) multiplies K-slice q of every tile by rows
+//     16 mh .. of X, and loads rows 8 mh .. 8 mh + 7 of the slice;
+//   * W and its E8M0 scales go global -> LDS with buffer_load ... lds (no VGPR staging), one DMA instruction per
+//     KiB of one weight row (two rows at K <= 4096); two tiles per workgroup are in flight (136 KiB per CU) while
+//     the previous one is multiplied; one barrier tells that a tile has landed, one that its slot may be refilled;
+//   * each wave keeps its K-slice of X (and of the X scales) resident in VGPRs for the whole kernel, in the 8-bit
+//     MFMA operand layout (bytes 16 g .. 16 g + 15 and 64 + 16 g .. of each K-step for lane group g); X reaches the
+//     registers through LDS, see the kernel;
+//   * v_mfma_scale_f32_16x16x128_f8f6f4 with mixed formats (W as FP4 first matrix, X as FP8 second matrix); W
+//     fragments are read from LDS (16-byte chunks XOR-swizzled by row: conflict free), the scale bytes of the
+//     lane's blocks are packed one register per four K-steps for op_sel to walk;
+//   * the 4 partial sums of a tile meet in LDS and two waves convert and store them while the next tiles stream.
+// K may be any multiple of 512 up to 8192: the kernel is instantiated for K-slices of 1024 (K <= 4096) and 2048
+// elements, and lanes whose bytes lie beyond K fetch nothing (their LDS bytes arrive as zeros, which multiply to
+// nothing), so a shorter K costs LDS reads and MFMAs of the padding but no memory traffic.  (A variant whose 8
+// waves all split K and need no barrier while streaming measured 5 - 25 % slower at every K and is gone.)
 #include <stdlib.h>
 
 #include "mx_common.h"
@@ -29,240 +32,20 @@ typedef __attribute__((address_space(3))) const v4i lds_cv4i;
 typedef __attribute__((address_space(3))) v4f lds_v4f;
 
 constexpr int kWaves = 8;
-constexpr int kBatch = 8;                      // tiles whose partial sums are kept in registers
 constexpr uint32_t kOob = 0x80000000u;         // beyond num_records of the descriptors built here
-
-template <int SPW, int MT>
-struct DecodeCfg {
-  static constexpr int LPR = SPW * 4;          // lanes (16-byte chunks) per row of a wave's W slice
-  static constexpr int RPI = 64 / LPR;         // rows per DMA instruction
-  static constexpr int ROWB = LPR * 16;        // bytes per row of the slice
-  static constexpr int SB = SPW * 4;           // scale bytes per row of the slice
-  static constexpr int SLOT = SPW * 1024 + 1024;
-  static constexpr int RING = kWaves * 2 * SLOT;
-  static constexpr int RED = kWaves * kBatch * MT * 64 * 16;
-  static constexpr int LDS_BYTES = RING > RED ? RING : RED;
-};
 
 __device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
-// SPW + 1 LDS-DMA loads of one tile: SPW KiB of W rows and the 16 x SB scale bytes behind them.
-// (A separate device function: the host pass of the compiler does not know the gfx950-only 16-byte
-// form of the builtin and must not meet it in the kernel body itself.)
-template <int SPW>
-__device__ inline void issue_tile_dma(const uint8_t* W, uint32_t wbytes, const uint8_t* S, uint32_t sbytes,
-                                      lds_u8* base, const uint32_t* woff, uint32_t soff, int wsoff, int ssoff) {
-  const __amdgpu_buffer_rsrc_t rsW = make_rsrc(W, wbytes), rsS = make_rsrc(S, sbytes);
-#pragma unroll
-  for (int j = 0; j < SPW; ++j)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsW, (lds_void*)(base + j * 1024), 16, woff[j], wsoff, 0, 0);
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsS, (lds_void*)(base + SPW * 1024), 16, soff, ssoff, 0, 0);
-}
-
-template <int XF, int SPW, int MT, typename OutT>
-__global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d) {
-  using Cf = DecodeCfg<SPW, MT>;
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
-  lds_u8* const smem = (lds_u8*)smem_generic;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r = lane & 15, gq = lane >> 4;
-  const int ksteps = d.K / 128;
-  const int s0 = wave * SPW;                   // first K-step of this wave's slice
-  lds_u8* const my = smem + wave * 2 * Cf::SLOT;
-
-  // ---- per-lane DMA offsets inside a tile --------------------------------------------------------------
-  const uint32_t wbytes = (uint32_t)((int64_t)d.N * d.ldw), sbytes = (uint32_t)((int64_t)d.N * d.ldws);
-  uint32_t woff[SPW];
-#pragma unroll
-  for (int j = 0; j < SPW; ++j) {
-    const int rr = j * Cf::RPI + lane / Cf::LPR, p = lane % Cf::LPR;
-    const int c = p ^ (rr & 15);               // chunk of the row that lives at LDS position p
-    woff[j] = (s0 + c / 4 < ksteps) ? (uint32_t)(rr * d.ldw + s0 * 64 + c * 16) : kOob;
-  }
-  uint32_t soff;
-  {
-    constexpr int LS = Cf::SB / 16;            // lanes per scale row
-    const int row = lane / LS, part = lane % LS;
-    soff = (row < 16 && s0 * 4 + part * 16 < d.K / 32) ? (uint32_t)(row * d.ldws + s0 * 4 + part * 16) : kOob;
-  }
-#define MX_ISSUE_TILE(tile, slot)                                                                        \
-  issue_tile_dma<SPW>(d.W, wbytes, d.Ws, sbytes, my + (slot) * Cf::SLOT, woff, soff, (tile) * 16 * (int)d.ldw, \
-                      (tile) * 16 * (int)d.ldws)
-
-  // tiles of this workgroup: blockIdx.x, + gridDim.x, ... -- at any moment the workgroups together read one
-  // contiguous window of W, which spreads evenly over the memory channels
-  const int tiles = d.N / 16;
-  const int G = gridDim.x, t_first = blockIdx.x;
-  const int t_count = t_first < tiles ? (tiles - t_first + G - 1) / G : 0;
-  if (t_count == 0) return;                    // uniform per workgroup
-
-  // ---- resident X fragments and scales ---------------------------------------------------------------
-  // All loads are issued unconditionally from clamped addresses (no branches, so they overlap), and
-  // before the W stream; they are put into operand form after the first W tiles have been requested.
-  v8i xf[MT][SPW];
-  int xs[MT][(SPW + 3) / 4];
-  v4i xlo[MT][SPW], xhi[MT][SPW], xsraw[MT][(SPW + 3) / 4];
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-    const int m = 16 * i + r;
-    const bool mok = m < d.M;
-    const uint8_t* const xrow = d.X + (int64_t)(mok ? m : 0) * d.ldx + gq * 16;
-    const uint8_t* const xsrow = d.Xs + (int64_t)(mok ? m : 0) * d.ldxs;
-#pragma unroll
-    for (int s = 0; s < SPW; ++s) {
-      const int ks = s0 + s < ksteps ? s0 + s : 0;
-      xlo[i][s] = *(const v4i*)(xrow + (int64_t)ks * 128);
-      xhi[i][s] = *(const v4i*)(xrow + (int64_t)ks * 128 + 64);
-    }
-#pragma unroll
-    for (int u = 0; u < (SPW + 3) / 4; ++u) {
-      // 16 scale bytes = the 4 blocks of K-steps s0 + 4u .. s0 + 4u + 3 (K is a multiple of 512)
-      const int ks = s0 + 4 * u < ksteps ? s0 + 4 * u : 0;
-      xsraw[i][u] = *(const v4i*)(xsrow + ks * 4);
-    }
-  }
-
-  // The X loads above are requested first: they are few, and queued behind the first W tiles they would
-  // hold back the first MFMA for as long as that burst takes to drain.  Now the W stream starts: the first
-  // two tiles of this workgroup.
-  __builtin_amdgcn_sched_barrier(0);
-  MX_ISSUE_TILE(t_first, 0);
-  if (t_count > 1) MX_ISSUE_TILE(t_first + G, 1);
-
-  __builtin_amdgcn_sched_barrier(0);
-  // X into the MFMA operand layout; rows beyond M and K-steps beyond K become zeros (scale 1.0)
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-    const bool mok = 16 * i + r < d.M;
-#pragma unroll
-    for (int s = 0; s < SPW; ++s) {
-      const bool ok = mok && s0 + s < ksteps;
-      const v4i lo = xlo[i][s], hi = xhi[i][s];
-      xf[i][s] = ok ? (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w} : (v8i){0, 0, 0, 0, 0, 0, 0, 0};
-    }
-#pragma unroll
-    for (int u = 0; u < (SPW + 3) / 4; ++u) {
-      uint32_t pk = 0;
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const bool ok = mok && s0 + 4 * u + t < ksteps;
-        const uint32_t byte = ok ? (((uint32_t)xsraw[i][u][t] >> (8 * gq)) & 0xFFu) : 127u;
-        pk |= byte << (8 * t);
-      }
-      xs[i][u] = (int)pk;
-    }
-  }
-
-  for (int tb = 0; tb < t_count; tb += kBatch) {   // local tile index; uniform per workgroup
-    const int nt = t_count - tb < kBatch ? t_count - tb : kBatch;
-    v4f acc[kBatch][MT];
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i)
-#pragma unroll
-      for (int m = 0; m < MT; ++m) acc[i][m] = (v4f){0.f, 0.f, 0.f, 0.f};
-
-    if (tb != 0) {                                      // the first batch was started above
-      MX_ISSUE_TILE(t_first + tb * G, 0);
-      if (nt > 1) MX_ISSUE_TILE(t_first + (tb + 1) * G, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i) {
-      if (i < nt) {                                     // uniform
-        // wait for tile i of the batch (and, the first time, for the older X loads); the SPW + 1 loads of
-        // tile i + 1 may stay in flight
-        if (i + 1 < nt) __builtin_amdgcn_s_waitcnt(0x0F70 | (SPW + 1));
-        else __builtin_amdgcn_s_waitcnt(0x0F70);
-        asm volatile("" ::: "memory");
-        lds_u8* const wt = my + (i & 1) * Cf::SLOT;
-        lds_u8* const st = wt + SPW * 1024;
-        v4i sc[Cf::SB / 16];
-#pragma unroll
-        for (int h = 0; h < Cf::SB / 16; ++h) sc[h] = *(lds_cv4i*)(st + r * Cf::SB + 16 * h);
-#pragma unroll
-        for (int s = 0; s < SPW; ++s) {
-          const v4i w = *(lds_cv4i*)(wt + r * Cf::ROWB + (((s * 4 + gq) ^ r) << 4));
-          const v8i wf = {w.x, w.y, w.z, w.w, 0, 0, 0, 0};
-          const int wscale = (int)((uint32_t)sc[s / 4][s % 4] >> (8 * gq));
-#pragma unroll
-          for (int m = 0; m < MT; ++m) {
-            if (s % 4 == 0)
-              acc[i][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[m][s], acc[i][m], MX_E2M1, XF, 0, wscale, 0, xs[m][s / 4]);
-            else if (s % 4 == 1)
-              acc[i][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[m][s], acc[i][m], MX_E2M1, XF, 0, wscale, 1, xs[m][s / 4]);
-            else if (s % 4 == 2)
-              acc[i][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[m][s], acc[i][m], MX_E2M1, XF, 0, wscale, 2, xs[m][s / 4]);
-            else
-              acc[i][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[m][s], acc[i][m], MX_E2M1, XF, 0, wscale, 3, xs[m][s / 4]);
-          }
-        }
-        // the slot is free again once its fragments are in registers: refill it two tiles ahead
-        __builtin_amdgcn_sched_barrier(0);
-        if (i + 2 < nt) MX_ISSUE_TILE(t_first + (tb + i + 2) * G, i & 1);
-      }
-    }
-
-    // ---- reduce the 8 K-slices: partial sums meet in LDS (the ring is idle now) -----------------------
-    __syncthreads();
-    lds_v4f* const red = (lds_v4f*)smem;
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i)
-#pragma unroll
-      for (int m = 0; m < MT; ++m)
-        if (i < nt) red[((wave * kBatch + i) * MT + m) * 64 + lane] = acc[i][m];
-    __syncthreads();
-    const bool vec_ok = (d.ldc % 4 == 0) && (((uintptr_t)d.C) % 16 == 0);
-    for (int it = tid; it < nt * MT * 64; it += kWaves * 64) {
-      const int i = it / (MT * 64), m = (it / 64) % MT, l = it & 63;
-      v4f sum = red[((0 * kBatch + i) * MT + m) * 64 + l];
-#pragma unroll
-      for (int w = 1; w < kWaves; ++w) sum += red[((w * kBatch + i) * MT + m) * 64 + l];
-      // lane (c, g) of tile i holds C[16 m + c][16 tile + 4 g + e], e = 0..3
-      const int row = 16 * m + (l & 15);
-      if (row < d.M) {
-        OutT* c = (OutT*)d.C + (int64_t)row * d.ldc + (t_first + (tb + i) * G) * 16 + 4 * (l >> 4);
-        if constexpr (sizeof(OutT) == 4) {
-          if (vec_ok) {
-            if (d.accumulate) sum += *(const v4f*)c;
-            *(v4f*)c = sum;
-          } else {
-            for (int e = 0; e < 4; ++e) c[e] = d.accumulate ? c[e] + sum[e] : sum[e];
-          }
-        } else {
-          if (vec_ok) {
-            if (d.accumulate) {
-              const uint2 old = *(const uint2*)c;
-              sum.x += bf16_to_f32((uint16_t)old.x); sum.y += bf16_to_f32((uint16_t)(old.x >> 16));
-              sum.z += bf16_to_f32((uint16_t)old.y); sum.w += bf16_to_f32((uint16_t)(old.y >> 16));
-            }
-            uint2 o;
-            o.x = (uint32_t)f32_to_bf16(sum.x) | ((uint32_t)f32_to_bf16(sum.y) << 16);
-            o.y = (uint32_t)f32_to_bf16(sum.z) | ((uint32_t)f32_to_bf16(sum.w) << 16);
-            *(uint2*)c = o;
-          } else {
-            for (int e = 0; e < 4; ++e)
-              c[e] = f32_to_bf16(d.accumulate ? bf16_to_f32(c[e]) + sum[e] : sum[e]);
-          }
-        }
-      }
-    }
-    if (tb + kBatch < t_count) __syncthreads();   // the next batch's DMA overwrites the reduction buffer
-  }
-#undef MX_ISSUE_TILE
-}
-
-// ---- variant for K = 4 * SPW * 128 (K = 4096, 8192) -------------------------------------------------------
-// The 8 waves are 4 K-slices x 2 halves of M (16 rows of X each), so a K-slice is twice as long as in
-// decode_kernel and, at K = 8192, one DMA instruction reads 1 KiB of ONE weight row instead of 512 bytes of
-// two (HBM streams long contiguous pieces measurably faster).  The two waves of a K-slice multiply the same
+// ---- configuration for K-slices of SPW K-steps (K <= 4 * SPW * 128) ------------------------------------------------
+// The two waves of a K-slice multiply the same
 // weight fragments by their own half of X, so a tile is shared through LDS: each of the two loads half of
 // the slice's rows, one workgroup barrier tells that a tile has landed and one that its slot may be
 // refilled.  LDS slot of a tile: [K-slice][row][slice bytes] (16-byte chunks XOR-swizzled by row), then
 // [row][K/32] scale bytes; two slots, i.e. two tiles in flight per workgroup.
 template <int SPW>
-struct Decode2Cfg {
+struct DecodeCfg {
   static constexpr int SLB = SPW * 64;            // bytes of a weight row inside one K-slice
   static constexpr int LPR = SLB / 16;            // lanes (16-byte chunks) per row of a slice
   static constexpr int RPI = 64 / LPR;            // rows per DMA instruction
@@ -294,14 +77,16 @@ struct Decode2Cfg {
 template <int SPW>
 __device__ inline void issue_tile_dma2(const uint8_t* W, uint32_t wbytes, const uint8_t* S, uint32_t sbytes,
                                        lds_u8* wdst, lds_u8* sdst, uint32_t row_off, uint32_t chunk_off, int rbase,
-                                       uint32_t soff, int wsoff, int ldw, int ssoff, bool with_scales) {
-  using Cf = Decode2Cfg<SPW>;
+                                       uint32_t soff, int wsoff, int ldw, int ssoff, bool with_scales,
+                                       uint32_t row_bytes) {
+  using Cf = DecodeCfg<SPW>;
   const __amdgpu_buffer_rsrc_t rsW = make_rsrc(W, wbytes), rsS = make_rsrc(S, sbytes);
 #pragma unroll
   for (int j = 0; j < Cf::WIW; ++j) {
     const int r0 = rbase + j * Cf::RPI;
+    const uint32_t off = chunk_off ^ (uint32_t)((r0 & 15) << 4);     // byte of the row this lane fetches
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsW, (lds_void*)(wdst + j * 1024), 16,
-                                             row_off + (chunk_off ^ (uint32_t)((r0 & 15) << 4)), wsoff + r0 * ldw, 0, 0);
+                                             off < row_bytes ? row_off + off : kOob, wsoff + r0 * ldw, 0, 0);
   }
   if (with_scales)   // uniform per wave
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsS, (lds_void*)sdst, 16, soff, ssoff, 0, 0);
@@ -309,12 +94,15 @@ __device__ inline void issue_tile_dma2(const uint8_t* W, uint32_t wbytes, const 
 
 // The 4 LDS-DMA loads of one staging round of a wave: 256 bytes of each of 16 consecutive rows of X (4 rows per
 // instruction), row rr to dst + rr * 256
-__device__ inline void issue_x_round(const uint8_t* X, uint32_t xbytes, lds_u8* dst, const uint32_t* voff, int soff0,
-                                     int ldx) {
+// (voff[j]: lane offset of instruction j; cb[j]: the byte inside the round's 256 that the lane fetches; bytes at or
+// beyond kleft, the end of the row, are not fetched and arrive as zeros)
+__device__ inline void issue_x_round(const uint8_t* X, uint32_t xbytes, lds_u8* dst, const uint32_t* voff, const int* cb,
+                                     int kleft, int soff0, int ldx) {
   const __amdgpu_buffer_rsrc_t rsX = make_rsrc(X, xbytes);
 #pragma unroll
   for (int j = 0; j < 4; ++j)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsX, (lds_void*)(dst + j * 1024), 16, voff[j], soff0 + 4 * j * ldx, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsX, (lds_void*)(dst + j * 1024), 16, cb[j] < kleft ? voff[j] : kOob,
+                                             soff0 + 4 * j * ldx, 0, 0);
 }
 __device__ inline void issue_xs_dma(const uint8_t* Xs, uint32_t bytes, lds_u8* dst, uint32_t voff, int soff) {
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(Xs, bytes);
@@ -322,8 +110,8 @@ __device__ inline void issue_xs_dma(const uint8_t* Xs, uint32_t bytes, lds_u8* d
 }
 
 template <int XF, int SPW, typename OutT>
-__global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d) {
-  using Cf = Decode2Cfg<SPW>;
+__global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d) {
+  using Cf = DecodeCfg<SPW>;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_generic[];
   lds_u8* const smem = (lds_u8*)smem_generic;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -341,7 +129,8 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
   // pieces of a row are XOR-swizzled by the row like the weight chunks, and the 16 rows a fragment read touches
   // sit in 16 different bank groups
   const int srow = wave * (64 / Cf::LS) + lane / Cf::LS;
-  const uint32_t soff = (uint32_t)(srow * d.ldws + (((lane % Cf::LS) ^ Cf::sswz(srow)) * 16));
+  const int spiece = ((lane % Cf::LS) ^ Cf::sswz(srow)) * 16;    // byte of the scale row this lane fetches
+  const uint32_t soff = spiece < d.K / 32 ? (uint32_t)(srow * d.ldws + spiece) : kOob;
   // Tiles of this workgroup: local tile i is tile t_first + i G (16 consecutive weight rows), so that the workgroups
   // together read one contiguous window of G tiles at a time.  Workgroup ids go round-robin over the 8 XCDs; XCD x
   // takes the x-th eighth of every window, so that every XCD reads from all address slices instead of always the
@@ -356,7 +145,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
     lds_u8* const base = smem + slot * Cf::SLOT;
     issue_tile_dma2<SPW>(d.W, wbytes, d.Ws, sbytes, base + q * (16 * Cf::SLB) + mh * Cf::WIW * 1024,
                          base + Cf::W_BYTES + wave * 1024, row_off, chunk_off, mh * Cf::WIW * Cf::RPI, soff,
-                         tile * 16 * (int)d.ldw, (int)d.ldw, tile * 16 * (int)d.ldws, with_scales);
+                         tile * 16 * (int)d.ldw, (int)d.ldw, tile * 16 * (int)d.ldws, with_scales, (uint32_t)(d.K / 2));
   };
 
   if (t_count == 0) return;                    // uniform per workgroup
@@ -380,18 +169,25 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
     lds_u8* const xsst = smem + Cf::XSCALE_OFF + wave * 1024;
     const uint32_t xbytes = (uint32_t)((int64_t)d.M * d.ldx);
     uint32_t xvo[4];                                  // lane offsets of the 4 DMA instructions of a round
+    int xcb[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) xvo[j] = (uint32_t)((lane >> 4) * d.ldx + (((lane & 15) ^ (4 * j + (lane >> 4))) << 4));
+    for (int j = 0; j < 4; ++j) {
+      xcb[j] = ((lane & 15) ^ (4 * j + (lane >> 4))) << 4;
+      xvo[j] = (uint32_t)((lane >> 4) * d.ldx + xcb[j]);
+    }
     const int xso = 16 * mh * (int)d.ldx + q * SPW * 128;
+    const int xk = d.K - q * SPW * 128;               // bytes of a row of X from the start of this wave's K-slice on
     // the wave's own X scales: 16 rows x SPW * 4 bytes, one instruction
     {
       constexpr int LPRS = SPW * 4 / 16;              // lanes per row
       const int srw = lane / LPRS;
+      const bool sok = srw < 16 && q * SPW * 4 + (lane % LPRS) * 16 < d.K / 32;
       issue_xs_dma(d.Xs, (uint32_t)((int64_t)d.M * d.ldxs), xsst,
-                   srw < 16 ? (uint32_t)(srw * d.ldxs + (lane % LPRS) * 16) : kOob, 16 * mh * (int)d.ldxs + q * SPW * 4);
+                   sok ? (uint32_t)(srw * d.ldxs + (lane % LPRS) * 16) : kOob, 16 * mh * (int)d.ldxs + q * SPW * 4);
     }
 #pragma unroll
-    for (int h = 0; h < Cf::XNB && h < XR; ++h) issue_x_round(d.X, xbytes, xst + h * 4096, xvo, xso + h * 256, (int)d.ldx);
+    for (int h = 0; h < Cf::XNB && h < XR; ++h)
+      issue_x_round(d.X, xbytes, xst + h * 4096, xvo, xcb, xk - h * 256, xso + h * 256, (int)d.ldx);
 #pragma unroll
     for (int h = 0; h < XR; ++h) {
       static_assert(Cf::XNB == 2, "wait counts below");
@@ -417,7 +213,8 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // round h + XNB (or the weight stream) overwrites the buffer
       if (h + Cf::XNB < XR)
-        issue_x_round(d.X, xbytes, xst + (h % Cf::XNB) * 4096, xvo, xso + (h + Cf::XNB) * 256, (int)d.ldx);
+        issue_x_round(d.X, xbytes, xst + (h % Cf::XNB) * 4096, xvo, xcb, xk - (h + Cf::XNB) * 256,
+                      xso + (h + Cf::XNB) * 256, (int)d.ldx);
     }
     __syncthreads();                                   // the weight slots overlap the other waves' staging areas
     if (t_count > 1) issue(1, 0);
@@ -531,35 +328,9 @@ __global__ __launch_bounds__(kWaves * 64) void decode2_kernel(const DecodeArgs d
 }
 
 template <int XF, int SPW, typename OutT>
-int launch_decode2_k(const DecodeArgs& d, int grid, hipStream_t stream) {
-  using Cf = Decode2Cfg<SPW>;
-  auto kern = decode2_kernel<XF, SPW, OutT>;
-  static int attr_done = 0;   // benign race: the attribute call is idempotent
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);
-    if (e != hipSuccess)
-      return set_error(MX_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", Cf::LDS_BYTES, hipGetErrorString(e));
-    attr_done = 1;
-  }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kWaves * 64), Cf::LDS_BYTES, stream, d);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return set_error(MX_ERR_LAUNCH, "decode2_kernel launch: %s", hipGetErrorString(e));
-  return MX_OK;
-}
-
-template <int XF>
-int launch_decode2_x(const DecodeArgs& d, int grid, hipStream_t stream) {
-  if (d.K == 8192)
-    return d.c_dtype == MX_F32 ? launch_decode2_k<XF, 16, float>(d, grid, stream)
-                               : launch_decode2_k<XF, 16, uint16_t>(d, grid, stream);
-  return d.c_dtype == MX_F32 ? launch_decode2_k<XF, 8, float>(d, grid, stream)
-                             : launch_decode2_k<XF, 8, uint16_t>(d, grid, stream);
-}
-
-template <int XF, int SPW, int MT, typename OutT>
 int launch_decode_k(const DecodeArgs& d, int grid, hipStream_t stream) {
-  using Cf = DecodeCfg<SPW, MT>;
-  auto kern = decode_kernel<XF, SPW, MT, OutT>;
+  using Cf = DecodeCfg<SPW>;
+  auto kern = decode_kernel<XF, SPW, OutT>;
   static int attr_done = 0;   // benign race: the attribute call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cf::LDS_BYTES);
@@ -573,19 +344,13 @@ int launch_decode_k(const DecodeArgs& d, int grid, hipStream_t stream) {
   return MX_OK;
 }
 
-template <int XF, int SPW, int MT>
-int launch_decode_t(const DecodeArgs& d, int grid, hipStream_t stream) {
-  return d.c_dtype == MX_F32 ? launch_decode_k<XF, SPW, MT, float>(d, grid, stream)
-                             : launch_decode_k<XF, SPW, MT, uint16_t>(d, grid, stream);
-}
-
 template <int XF>
 int launch_decode_x(const DecodeArgs& d, int grid, hipStream_t stream) {
-  const int ksteps = d.K / 128;
-  const bool one = d.M <= 16;
-  if (ksteps <= kWaves * 4)
-    return one ? launch_decode_t<XF, 4, 1>(d, grid, stream) : launch_decode_t<XF, 4, 2>(d, grid, stream);
-  return one ? launch_decode_t<XF, 8, 1>(d, grid, stream) : launch_decode_t<XF, 8, 2>(d, grid, stream);
+  if (d.K > 4096)
+    return d.c_dtype == MX_F32 ? launch_decode_k<XF, 16, float>(d, grid, stream)
+                               : launch_decode_k<XF, 16, uint16_t>(d, grid, stream);
+  return d.c_dtype == MX_F32 ? launch_decode_k<XF, 8, float>(d, grid, stream)
+                             : launch_decode_k<XF, 8, uint16_t>(d, grid, stream);
 }
 
 }  // namespace
@@ -607,13 +372,7 @@ int launch_gemm_decode(const DecodeArgs& d, hipStream_t stream) {
   const int tiles = d.N / 16;
   const int grid = tiles < 256 ? tiles : 256;
   if (grid == 0) return MX_OK;
-  // the two-halves variant where its K-slices are whole (1024 or 2048 elements); with M <= 16 its second
-  // half of the waves multiplies zeros but still carries half of the DMA, and it measures 1 - 4 % faster than
-  // the 8-slice kernel there too (M = 1: 28.2 against 29.5 us on the 28672 x 8192 weights)
-  if (d.K == 8192 || d.K == 4096)
-    return d.x_fmt == MX_E4M3 ? launch_decode2_x<MX_E4M3>(d, grid, stream) : launch_decode2_x<MX_E5M2>(d, grid, stream);
-  if (d.x_fmt == MX_E4M3) return launch_decode_x<MX_E4M3>(d, grid, stream);
-  return launch_decode_x<MX_E5M2>(d, grid, stream);
+  return d.x_fmt == MX_E4M3 ? launch_decode_x<MX_E4M3>(d, grid, stream) : launch_decode_x<MX_E5M2>(d, grid, stream);
 }
 
 }  // namespace mx

@@ -11,7 +11,9 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("M,N,K", [(32, 256, 1024), (7, 1792, 2048), (16, 48, 512), (32, 4096, 8192), (1, 16, 4096),
                                    (17, 4176, 4096), (29, 12320, 8192), (32, 16, 8192), (24, 36864, 4096),
-                                   (8, 20480, 4096), (16, 16400, 8192)])
+                                   (8, 20480, 4096), (16, 16400, 8192),
+                                   # K that ends inside the kernel's K-slices: lanes beyond K fetch nothing
+                                   (32, 1792, 7168), (9, 528, 5120), (32, 272, 3072), (16, 64, 1536), (32, 4112, 6144)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=str)
 def test_decode_kernel(ct, dev, M, N, K, out_dtype):
     x = randn_operand(M, K, O.E4M3, 81, dev)
