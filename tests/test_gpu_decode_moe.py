@@ -155,7 +155,10 @@ def test_moe_pipeline_matches_oracle(ct, dev, kernel, tile_m, w_fmt):
     """cutile_moe_scaled (structure of cutile_moe, samples/MoE.py:197-288) against the oracle's
     moe_forward.  The intermediate is rounded to bf16 and re-quantised on both sides, so a last-bit
     difference of the first GEMM can move single elements by one E4M3 step: tolerance 2e-2 relative
-    Frobenius (the reference's own MoE check uses atol 1e-1, samples/MoE.py:462)."""
+    Frobenius (the reference's own MoE check uses atol 1e-1, samples/MoE.py:462).
+    PARITY UNPINNED: the reference has no block-scaled MoE and no test of one; this composition (re-quantising the
+    SiLU-gated intermediate) is checked against the oracle's own per-expert formula only.  The grouped GEMM it is
+    built from has its own gate against the dense per-expert reference (test_grouped_gemm_*, 1e-3 / 8e-3)."""
     T, H, F, E, topk = 96, 256, 128, 4, 2
     rng = np.random.default_rng(3)
     hq, hs = O.block_quantize(rng.standard_normal((T, H)).astype(np.float32), 32, O.E4M3, "floor")
