@@ -111,3 +111,27 @@ def test_moe_shape_properties(ct, dev):
         ref = a[pick[:, 0]] @ w.T
         got = c[torch.from_numpy(pick[:, 0]).to(dev), torch.from_numpy(pick[:, 1]).to(dev)].float().cpu()
         assert O.rel_fro(got, ref) < 8e-3
+
+
+@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (12288, 4096, 2560)])
+def test_reference_bench_shapes_swizzled(ct, dev, M, N, K):
+    """The other two shapes of the reference's swizzled-scale benchmark (test/bench_matmul.py:421-425, operands as
+    in :497-499: E4M3, block 32, both scale tensors in swizzle_32_4_4 order, fp32 out), checked before any timing as
+    that benchmark does: swizzled and 2-D scales give the same bits, two independent kernels give the same bits, and
+    the result matches the oracle (every output of 1024^3; 96 sampled rows of the large one)."""
+    a_q, a_s = _operand(ct, dev, M, K, O.E4M3, 401)
+    b_q, b_s = _operand(ct, dev, N, K, O.E4M3, 402)
+    a_sw, b_sw = ct.swizzle_32_4_4(a_s), ct.swizzle_32_4_4(b_s)
+    c = ct.block_scaled_matmul(a_q, a_sw, b_q.T, b_sw, out_dtype=torch.float32)
+    c_2d = ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, out_dtype=torch.float32)
+    assert torch.equal(c.view(torch.int32), c_2d.view(torch.int32))
+    c_ref = ct.block_scaled_matmul(a_q, a_sw, b_q.T, b_sw, out_dtype=torch.float32, kernel="mfma128")
+    assert torch.equal(c.view(torch.int32), c_ref.view(torch.int32))
+    a = _dequant_cpu(a_q, a_s, O.E4M3)
+    b = _dequant_cpu(b_q, b_s, O.E4M3)
+    rows = torch.arange(M) if M <= 1024 else torch.from_numpy(np.random.default_rng(11).choice(M, 96, replace=False))
+    ref = a[rows].double() @ b.double().T
+    got = c[rows.to(dev)].double().cpu()
+    # fp32 accumulation of K exact products inside and across the MFMA instructions, against float64
+    assert O.rel_fro(got, ref) < 1e-4
+    assert torch.allclose(got, ref, atol=1e-4 * float(ref.abs().max()), rtol=1e-3)
