@@ -62,7 +62,10 @@ __device__ __attribute__((noinline)) void write_tile_checked(AccTile t, OutT* Cp
   }
 }
 
-template <class C, typename OutT, bool GROUPED, int TEAM>
+// KTAIL: K is not a whole number of stages (or there is a single stage): the 16-byte chunks beyond the end of K are
+// masked lane by lane at issue time.  Without it the loads take their precomputed offsets as they are, which keeps a
+// compare and a select per DMA instruction out of the memory phase.
+template <class C, typename OutT, bool GROUPED, int TEAM, bool KTAIL>
 __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, const int wn,
                                         const int lane, const TileWalk& walk) {
   using P = PP<C>;
@@ -166,7 +169,9 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     const int klim = sl < nstages ? Kb_a - ka : 0;   // bytes of this stage's rows that exist
 #pragma unroll
     for (int q = 0; q < AL; ++q) {
-      const uint32_t v = a_col0 >= klim ? kOobOffset : a_voff[q];
+      // (without a K tail a stage at or beyond nstages is only ever requested once the walk has no further tile, and
+      // then every offset is out of range already)
+      const uint32_t v = (KTAIL && a_col0 >= klim) ? kOobOffset : a_voff[q];
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_void*)(base + q * 4096), 16, v, ka, 0, 0);
     }
   };
@@ -178,7 +183,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
 #pragma unroll
       for (int q = 0; q < BL; ++q) {
         const int col = b_col(q);
-        const uint32_t v = col >= klim ? kOobOffset : b_voff[q];
+        const uint32_t v = (KTAIL && col >= klim) ? kOobOffset : b_voff[q];
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(base + q * 1024), 16, v, kb, 0, 0);
       }
     }
@@ -438,10 +443,21 @@ __global__ __launch_bounds__(512) void gemm_pp_kernel(const GemmArgs g) {
 
   const TileWalk walk = make_tile_walk(g.M, g.N);
   if (walk.first >= walk.end) return;   // cannot happen with the grids the launcher picks
-  if (wave < 4)
-    pp_body<C, OutT, GROUPED, 0>(g, smem, wave, lane, walk);
-  else
-    pp_body<C, OutT, GROUPED, 1>(g, smem, wave - 4, lane, walk);
+  const int ksteps = (g.K + 127) / 128;
+  // (uniform.  The MXFP4 instance keeps the one masked body: with two bodies in the kernel the register allocator
+  // spills in its stage loop.)
+  const bool ktail = C::KSUB != 1 || g.K % 128 != 0 || ksteps < 2;
+  if (ktail) {
+    if (wave < 4)
+      pp_body<C, OutT, GROUPED, 0, true>(g, smem, wave, lane, walk);
+    else
+      pp_body<C, OutT, GROUPED, 1, true>(g, smem, wave - 4, lane, walk);
+  } else if constexpr (C::KSUB == 1) {
+    if (wave < 4)
+      pp_body<C, OutT, GROUPED, 0, false>(g, smem, wave, lane, walk);
+    else
+      pp_body<C, OutT, GROUPED, 1, false>(g, smem, wave - 4, lane, walk);
+  }
 }
 
 template <class C, typename OutT, bool GROUPED>
