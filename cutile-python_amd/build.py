@@ -36,12 +36,12 @@ def _newer(src: pathlib.Path, obj: pathlib.Path) -> bool:
 
 
 def _flags_changed() -> bool:
-    """True (and the stamp is rewritten) when the objects on disk were built with other flags."""
+    """True when the objects on disk were built with other flags (the stamp is removed until the next build has
+    compiled every object, so a failed build never leaves old objects looking current)."""
     stamp = OBJ / "flags.txt"
-    want = " ".join(FLAGS)
-    if stamp.exists() and stamp.read_text() == want:
+    if stamp.exists() and stamp.read_text() == " ".join(FLAGS):
         return False
-    stamp.write_text(want)
+    stamp.unlink(missing_ok=True)
     return True
 
 
@@ -62,6 +62,7 @@ def build(force: bool = False, jobs: int | None = None) -> pathlib.Path:
     jobs = jobs or min(len(SOURCES), os.cpu_count() or 4, 8)
     with ThreadPoolExecutor(jobs) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), SOURCES))
+    (OBJ / "flags.txt").write_text(" ".join(FLAGS))
     cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(OUT), *map(str, objs)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:

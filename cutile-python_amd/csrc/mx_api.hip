@@ -691,6 +691,7 @@ int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W,
   if ((num_valid_ids + num_token_replicas - 1) / num_token_replicas > T)
     return set_error(MX_ERR_SHAPE, "num_valid_ids / num_token_replicas exceeds the rows of A");
   if (num_slots == 0 || N == 0) return MX_OK;
+  if (E <= 0 || E > 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "W must hold at least one expert");
   if (A->dtype == MX_E2M1 && A->packed_dim != 1) return set_error(MX_ERR_LAYOUT, "A must be packed along K");
   if (W->dtype == MX_E2M1 && W->packed_dim != 2) return set_error(MX_ERR_LAYOUT, "W must be packed along K");
 
@@ -730,6 +731,7 @@ int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W,
     g.c_sm = C->stride[0]; g.c_sn = C->stride[1];
     g.sorted_token_ids = sorted_token_ids; g.sorted_expert_ids = sorted_expert_ids; g.topk_weights = topk_weights;
     g.tile_m = tile_m; g.replicas = num_token_replicas; g.num_valid_ids = num_valid_ids; g.num_slots = num_slots;
+    g.num_experts = (int32_t)E;
     return launch_gemm_generic(g, (hipStream_t)stream);
   }
 
@@ -762,6 +764,7 @@ int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W,
   g.a_fmt = A->dtype; g.b_fmt = W->dtype; g.c_dtype = C->dtype; g.accumulate = o.accumulate;
   g.sorted_token_ids = sorted_token_ids; g.sorted_expert_ids = sorted_expert_ids; g.topk_weights = topk_weights;
   g.tile_m = tile_m; g.replicas = num_token_replicas; g.num_valid_ids = num_valid_ids;
+  g.num_experts = (int32_t)E;
   g.b_expert_stride = W->stride[0];
   g.bs_expert_stride = mx_packed_scale_bytes(N, K) / 4;
   g.a_rows = T;

@@ -90,6 +90,7 @@ struct GemmArgs {
   const int32_t* sorted_expert_ids;
   const float* topk_weights;
   int32_t tile_m, replicas;
+  int32_t num_experts;       // entries of sorted_expert_ids are clamped to [0, num_experts)
   int64_t num_valid_ids;
   int64_t b_expert_stride;   // bytes between experts in B
   int64_t bs_expert_stride;  // dwords between experts in Bs
@@ -131,7 +132,7 @@ struct GenericArgs {
   int32_t as_layout, bs_layout;         // MX_SCALE_2D or MX_SCALE_SWIZZLE_32_4_4
   // grouped extension
   const int32_t* sorted_token_ids; const int32_t* sorted_expert_ids; const float* topk_weights;
-  int32_t tile_m, replicas; int64_t num_valid_ids; int64_t num_slots;
+  int32_t tile_m, replicas, num_experts; int64_t num_valid_ids; int64_t num_slots;
   int64_t b_se, bs_se;                  // expert strides (bytes)
 };
 int launch_gemm_generic(const GenericArgs& g, hipStream_t stream);

@@ -155,8 +155,9 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
   // its operand registers out of its own staging area.  (Loading the operand layout straight from memory, 16 rows
   // x 64 bytes per instruction and every workgroup the same 264 KiB, keeps the texture-address unit and L2 busy for
   // 6 us at the 32 x 8192 activations; this way the 256 KiB cross the CU's 64-byte/clock memory port in 3 us.)  A round
-  // is two K-steps: 16 rows x 256 bytes per wave, 16-byte chunks XOR-swizzled by row; two rounds are in flight.  Rows
-  // at or beyond M are out of range of the descriptor and arrive as zeros (scale byte 0 = 2^-127).
+  // is two K-steps: 16 rows x 256 bytes per wave, 16-byte chunks XOR-swizzled by row; two rounds are in flight.  Lanes
+  // whose row is at or beyond M fetch nothing (offset beyond the descriptor) and their bytes arrive as zeros (scale
+  // byte 0 = 2^-127).
   // The DMA of tile 0 is requested first: the memory pipe returns data in request order for the whole CU, so X
   // arrives behind it, but HBM has something to do meanwhile (0.7 us faster than staging X first); with both first
   // tiles in flight there would be no room in LDS to stage X.
@@ -173,7 +174,9 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       xcb[j] = ((lane & 15) ^ (4 * j + (lane >> 4))) << 4;
-      xvo[j] = (uint32_t)((lane >> 4) * d.ldx + xcb[j]);
+      // the row term 16 mh + 4 j of the address travels in the instruction's scalar offset, which the descriptor's
+      // range check does not see: a lane whose row is at or beyond M is masked here instead
+      xvo[j] = 16 * mh + 4 * j + (lane >> 4) < d.M ? (uint32_t)((lane >> 4) * d.ldx + xcb[j]) : kOob;
     }
     const int xso = 16 * mh * (int)d.ldx + q * SPW * 128;
     const int xk = d.K - q * SPW * 128;               // bytes of a row of X from the start of this wave's K-slice on
@@ -181,7 +184,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
     {
       constexpr int LPRS = SPW * 4 / 16;              // lanes per row
       const int srw = lane / LPRS;
-      const bool sok = srw < 16 && q * SPW * 4 + (lane % LPRS) * 16 < d.K / 32;
+      const bool sok = srw < 16 && 16 * mh + srw < d.M && q * SPW * 4 + (lane % LPRS) * 16 < d.K / 32;
       issue_xs_dma(d.Xs, (uint32_t)((int64_t)d.M * d.ldxs), xsst,
                    sok ? (uint32_t)(srw * d.ldxs + (lane % LPRS) * 16) : kOob, 16 * mh * (int)d.ldxs + q * SPW * 4);
     }

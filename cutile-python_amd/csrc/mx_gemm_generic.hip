@@ -51,7 +51,8 @@ __global__ __launch_bounds__(256) void generic_kernel(const GenericArgs g) {
     if (id < 0 || id >= g.num_valid_ids) return;
     arow = id / g.replicas;
     crow = id;
-    const int e = g.sorted_expert_ids[mrow / g.tile_m];
+    int e = g.sorted_expert_ids[mrow / g.tile_m];
+    e = e < 0 ? 0 : (e >= g.num_experts ? g.num_experts - 1 : e);   // never outside W
     boff = (int64_t)e * g.b_se;
     bsoff = (int64_t)e * g.bs_se;
     if (g.topk_weights) w = g.topk_weights[id];

@@ -71,7 +71,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, lds_u8* const smem,
   const int KQ = (ksteps + 3) / 4;
 
   int expert = 0;
-  if constexpr (GROUPED) expert = g.sorted_expert_ids[m0 / g.tile_m];
+  if constexpr (GROUPED) {
+    expert = g.sorted_expert_ids[m0 / g.tile_m];
+    expert = expert < 0 ? 0 : (expert >= g.num_experts ? g.num_experts - 1 : expert);
+  }
 
   const uint8_t* Bbase = g.B + (GROUPED ? (int64_t)expert * g.b_expert_stride : 0);
   const __amdgpu_buffer_rsrc_t rsA = make_rsrc(g.A, (uint32_t)(g.a_rows * g.lda));

@@ -109,10 +109,9 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     for (int j = 0; j < 4; ++j) sb[j] = Bs1[(int64_t)idx16 * 4 + 16 * (j & 1) + 2 * (j >> 1)];
   };
   bool fetch_valid = true;   // false once the walk has no further tile: loads become zero-fill no-ops
-  // grouped: this team's 128 rows of the tile are all alignment padding (the padding of an expert's block is its
-  // tail, and blocks are whole tiles, so it is enough to look at the first row of the half).  Such a half has
-  // nothing to multiply: its fragment reads and MFMAs are skipped, which is what makes a half-filled tile cost
-  // about as much as a 128-row tile would.
+  // grouped: none of this team's 128 slots of the tile holds a routed row (every slot is looked at: two per lane,
+  // then a vote, so a sentinel in front of valid ids does not hide them).  Such a half has nothing to multiply:
+  // its fragment reads and MFMAs are skipped.
   bool skip_cur = false, skip_nxt = false;
   auto set_fetch_tile = [&](int lid) {
     fetch_valid = lid < walk.end;
@@ -120,15 +119,23 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     if (fetch_valid) walk.origin(lid, m0, n0);
     if constexpr (GROUPED) {
       skip_nxt = false;
-      if (fetch_valid && m0 + wm0 < g.M) {
-        const int id0 = g.sorted_token_ids[m0 + wm0];
-        skip_nxt = id0 < 0 || id0 >= g.num_valid_ids;
-      } else if (fetch_valid) {
-        skip_nxt = true;
+      if (fetch_valid) {
+        bool any = false;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int m = m0 + wm0 + 64 * u + lane;
+          const int id = m < g.M ? g.sorted_token_ids[m] : -1;
+          any = any || (id >= 0 && id < g.num_valid_ids);
+        }
+        skip_nxt = __builtin_amdgcn_ballot_w64(any) == 0;
       }
     }
     int expert = 0;
-    if constexpr (GROUPED) expert = g.sorted_expert_ids[m0 / g.tile_m];
+    if constexpr (GROUPED) {
+      // an id outside [0, experts) would move the descriptor's base past W, where the range check no longer helps
+      expert = g.sorted_expert_ids[m0 / g.tile_m];
+      expert = expert < 0 ? 0 : (expert >= g.num_experts ? g.num_experts - 1 : expert);
+    }
     const uint8_t* Bbase = g.B + (GROUPED ? (int64_t)expert * g.b_expert_stride : 0);
     rsB = make_rsrc(Bbase, (uint32_t)((int64_t)g.N * g.ldb));
 #pragma unroll

@@ -138,7 +138,10 @@ __device__ __forceinline__ void pp32_body(const GemmArgs& g, lds_u8* const smem,
     int m0 = 0, n0 = 0;
     if (fetch_valid) walk.origin(lid, m0, n0);
     int expert = 0;
-    if constexpr (GROUPED) expert = g.sorted_expert_ids[m0 / g.tile_m];
+    if constexpr (GROUPED) {
+      expert = g.sorted_expert_ids[m0 / g.tile_m];
+      expert = expert < 0 ? 0 : (expert >= g.num_experts ? g.num_experts - 1 : expert);
+    }
     const uint8_t* Bbase = g.B + (GROUPED ? (int64_t)expert * g.b_expert_stride : 0);
     rsB = make_rsrc(Bbase, (uint32_t)((int64_t)g.N * g.ldb));
 #pragma unroll

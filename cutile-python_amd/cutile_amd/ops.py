@@ -174,6 +174,9 @@ class _ScaleCache:
                 self._entries.move_to_end(key)
                 if e[4] != stream.cuda_stream:
                     stream.wait_event(e[3])          # the re-layout ran on another stream
+                    # the copy belongs to the allocator pool of that stream: tell it that this one reads it too,
+                    # so that dropping the entry while this stream's GEMM is in flight does not recycle the block
+                    e[2].data.record_stream(stream)
                 return e[2]
         packed = pack_scales(s, transposed=transposed)
         if torch.cuda.is_current_stream_capturing():

@@ -5,9 +5,13 @@
  * point enqueues work on the given hipStream_t (passed as void*; NULL = the null stream) and
  * returns without synchronising.  Return value: 0 on success, a negative MX_ERR_* otherwise; the
  * message of the last error on the calling thread is available from mx_last_error().
- * The library keeps no mutable global state besides that thread-local string, so calls from
- * several host threads are safe.  Nothing here allocates device memory: any workspace is passed
- * in by the caller.
+ * Calls from several host threads are safe: besides that thread-local string the library's only
+ * mutable state is set-once caches (the per-device address of the static scratch of mx_gemm_static,
+ * per-kernel "launch attribute set" flags and the CU count of the device that was current at the
+ * first launch; a racing thread stores the same value).  The library serves one device model
+ * (MI355X): with several GPUs in one process all of them are assumed to have the same CU count.
+ * Nothing here allocates device memory: any workspace is passed in by the caller, except for
+ * mx_gemm_static, whose scratch is a fixed buffer inside the library's device image.
  *
  * Each declaration names the reference interface (NVIDIA cuTile Python, path:line) it stands in for.
  */
@@ -174,8 +178,11 @@ MX_API int mx_gemm_static(const mx_tensor* A, const mx_tensor* A_scale, const mx
  * A list of independent block-scaled products C[i] = A[i] x B[i] (problem sizes may all differ), the
  * block-scaled counterpart of grouped_matmul_kernel(As, Bs, Cs, ...), test/kernels/group_gemm.py:10-38.
  * The descriptor arrays hold `count` entries each; every problem follows the rules of mx_gemm.  All problems are
- * validated first: on error the index of the failing problem is part of mx_last_error() and nothing has been
- * enqueued.  Problems that mx_gemm would give to its 128 x 128 one-tile kernel (the small and medium ones, which
+ * validated first: on error the index of the failing problem is part of mx_last_error().  A problem that is
+ * refused by these checks (descriptors, shapes, dtypes, layouts, workspace) leaves nothing enqueued; a problem of the
+ * kinds listed below as "the others" can still be refused by the kernel it is sent to (for example a forced kernel
+ * that does not take its shape), after the problems in front of it have been enqueued.  The C tensors of a list must
+ * not overlap: its problems run side by side, not in list order.  Problems that mx_gemm would give to its 128 x 128 one-tile kernel (the small and medium ones, which
  * is what such lists hold) run the way the reference's kernel does: one launch re-lays up to 64 scale
  * tensors, and one launch of persistent workgroups walks the concatenated tile list of up to 32 problems of one
  * element-format pair and output type (tile_idx += number of workgroups).  The others (large problems for the
@@ -212,7 +219,9 @@ MX_API int mx_bench_gemm(int32_t nsets, const mx_tensor* A, const mx_tensor* A_s
  *   A  [T,K] tokens, As [T,K/32];  W [E,N,K] (K contiguous), Ws [E,N,K/32];  C [T*replicas? ,N]:
  *   for every slot p of sorted_token_ids with id = sorted_token_ids[p] < num_valid_ids:
  *       C[id,:] = (A[id / num_token_replicas,:] * As) @ (W[e,:,:] * Ws[e]).T * (w ? w[id] : 1)
- *   where e = sorted_expert_ids[p / tile_m].  Slots holding the sentinel are skipped.
+ *   where e = sorted_expert_ids[p / tile_m] (an entry outside [0, E) is clamped into that range, so nothing
+ *   outside W is ever read; its rows are unspecified).  Slots holding the sentinel are skipped, wherever they
+ *   sit in a tile.
  *   topk_weights may be NULL (no routed-weight multiply).
  * Workspace: mx_gemm_grouped_workspace_bytes().
  */

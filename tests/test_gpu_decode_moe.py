@@ -149,6 +149,38 @@ def test_grouped_gemm_routed_weight_replicas1_and_padded_ids(ct, dev, kernel):
         assert O.rel_fro(C3.float().cpu(), ref * wts.reshape(-1, 1)) < 8e-3
 
 
+@pytest.mark.parametrize("kernel", ["generic", "mfma128", "mfma256", "pingpong", "pingpong32"])
+def test_grouped_gemm_sentinels_anywhere_and_expert_ids_out_of_range(ct, dev, kernel):
+    """Caller-built index arrays: the sentinel may sit in any slot of a tile (here in the first slot of each
+    128-row half, with routed rows behind it), as fused_moe_kernel masks slot by slot
+    (test/kernels/fused_moe.py:40-47); blocks whose expert id lies outside [0, E) hold only sentinels and must not
+    make the kernel read outside W."""
+    T, K, N, E, topk = 200, 256, 512, 4, 1
+    a, W, Ws, ids, ref = _moe_case(T, K, N, E, topk, 97, dev)
+    flat = ids.reshape(-1).numpy()
+    sent = T * topk
+    slots, experts = [], []
+    for e in range(E):
+        mine = np.nonzero(flat == e)[0].astype(np.int32)
+        assert 2 <= len(mine) <= 254
+        half = len(mine) // 2
+        block = np.full(256, sent, dtype=np.int32)
+        block[1:1 + half] = mine[:half]                      # slot 0 stays a sentinel
+        block[129:129 + len(mine) - half] = mine[half:]      # and so does slot 128
+        slots.append(block)
+        experts.append(e)
+    for bad in (E + 5, -3, 2 ** 30):
+        slots.append(np.full(256, sent, dtype=np.int32))
+        experts.append(bad)
+    sid = torch.from_numpy(np.concatenate(slots)).to(dev)
+    eid = torch.tensor(experts, dtype=torch.int32, device=dev)
+    for out_dtype, tol in ((torch.float32, 1e-3), (torch.bfloat16, 8e-3)):
+        C = torch.full((T * topk, N), float("nan"), device=dev, dtype=out_dtype)
+        ct.invoke_fused_moe_scaled(a.storage, a.scale_t, W, Ws, C, None, sid, eid, False, topk, 256, kernel=kernel)
+        torch.cuda.synchronize()
+        assert O.rel_fro(C.float().cpu(), ref) <= tol
+
+
 @pytest.mark.parametrize("kernel,tile_m", [("auto", 128), ("auto", 256), ("generic", 16)])
 @pytest.mark.parametrize("w_fmt", [O.E4M3, O.E2M1])
 def test_moe_pipeline_matches_oracle(ct, dev, kernel, tile_m, w_fmt):

@@ -320,6 +320,24 @@ def test_cached_scale_relayout(ct, dev):
         c5 = ct.block_scaled_matmul(a.storage, a.scale_t, b.storage.T, b.scale_t.T, cache_scales=True)
     s.synchronize()
     assert torch.equal(c5, c4)
+    # the entry is dropped while a GEMM on the other stream still reads the cached copy: the copy's block must not
+    # be handed out again before that GEMM is done (new allocations of the same size right behind the clear)
+    big_a = randn_operand(2048, 4096, O.E4M3, 73, dev)
+    big_b = randn_operand(2048, 4096, O.E4M3, 74, dev)
+    want = ct.block_scaled_matmul(big_a.storage, big_a.scale_t, big_b.storage.T, big_b.scale_t.T)
+    ct.block_scaled_matmul(big_a.storage, big_a.scale_t, big_b.storage.T, big_b.scale_t.T, cache_scales=True)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        for _ in range(4):                   # a few launches deep, so the last one is still queued at the clear
+            c7 = ct.block_scaled_matmul(big_a.storage, big_a.scale_t, big_b.storage.T, big_b.scale_t.T,
+                                        cache_scales=True)
+    ct.clear_scale_cache()
+    junk = [torch.full((ct.lib().mx_packed_scale_bytes(2048, 4096),), 0xFF, dtype=torch.uint8, device=dev)
+            for _ in range(4)]
+    s.synchronize()
+    torch.cuda.synchronize()
+    assert torch.equal(c7, want)
+    del junk
     # a problem of the general kernel (row-major B) ignores the cache
     b_rm = b.storage.T.contiguous()
     ref = ct.block_scaled_matmul(a.storage, a.scale_t, b_rm, b.scale_t.T)

@@ -40,12 +40,27 @@ def _both(ct, dev, a, b, out_dtype, kernel="auto", split_k=0, fill=None):
     return outs
 
 
+def _hostile_scratch(ct, dev):
+    """Leaves NaN everywhere a later call could read the static scratch: static calls whose scale bytes are all
+    0xFF (re-laid scales of 0xFF, then split-K partial products that are NaN)."""
+    def nan_operand(rows, K):
+        q = torch.zeros((rows, K), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+        s = torch.full((rows, K // 32), 0xFF, dtype=torch.uint8, device=dev).view(torch.float8_e8m0fnu)
+        return q, s
+    for (m, n, k), split in (((4096, 4096, 4096), 0), ((64, 256, 8192), 4)):
+        a_q, a_s = nan_operand(m, k)
+        b_q, b_s = nan_operand(n, k)
+        c = ct.block_scaled_matmul(a_q, a_s, b_q.T, b_s.T, static_scratch=True, split_k=split)
+        assert torch.isnan(c).all()
+
+
 def test_static_scratch_matches_workspace_entry_point(ct, dev):
     assert ct.lib().mx_static_scratch_bytes() == 8 << 20
+    hostile = lambda: _hostile_scratch(ct, dev)
     # first call: 4 x 4 tiles of 256 x 256 ... a large re-layout that fills a good part of the scratch
     a1 = randn_operand(3072, 2048, O.E4M3, 601, dev)
     b1 = randn_operand(3072, 2048, O.E4M3, 602, dev)
-    s1, w1 = _both(ct, dev, a1, b1, torch.bfloat16)
+    s1, w1 = _both(ct, dev, a1, b1, torch.bfloat16, fill=hostile)
     assert torch.equal(s1.view(torch.int16), w1.view(torch.int16))
     # second call, smaller and ragged, right behind it on the same scratch
     a2 = randn_operand(300, 160, O.E4M3, 603, dev)
@@ -56,10 +71,10 @@ def test_static_scratch_matches_workspace_entry_point(ct, dev):
     # third: split-K (per-slice scales and fp32 partial products in the scratch), then the first shape again
     a3 = randn_operand(64, 8192, O.E4M3, 605, dev)
     b3 = randn_operand(256, 8192, O.E4M3, 606, dev)
-    s3, w3 = _both(ct, dev, a3, b3, torch.float32)
+    s3, w3 = _both(ct, dev, a3, b3, torch.float32, fill=hostile)
     assert torch.equal(s3, w3)
     assert O.rel_fro(s3.cpu(), oracle_matmul(a3, b3)) <= 1e-3
-    s1b, _ = _both(ct, dev, a1, b1, torch.bfloat16)
+    s1b, _ = _both(ct, dev, a1, b1, torch.bfloat16, fill=hostile)
     assert torch.equal(s1b.view(torch.int16), w1.view(torch.int16))
     assert O.rel_fro(s1b[:64].float().cpu(), oracle_matmul(a1, b1)[:64]) <= 8e-3
 
