@@ -227,7 +227,8 @@ def bench_gemm(ct, O, dev, M, N, K, fmt, dist, steps, warmup, check, kernel="aut
     t_step = _time_wall(step, steps, warmup)
     # kernel alone: scales pre-packed, one pair of HIP events per launch recorded by the library's own timing
     # entry point (mx_bench_gemm) on the launch stream, operand sets rotated
-    packed = [(s[0], ct.pack_scales(s[1]), s[2].T, ct.pack_scales(s[3]), s[4]) for s in sets]
+    packed = [(s[0], ct.pack_scales(s[1], operand="a", kernel=kernel), s[2].T, ct.pack_scales(s[3], operand="b", kernel=kernel),
+               s[4]) for s in sets]
     state = {"warm": False}
 
     def batch(k):
@@ -291,7 +292,7 @@ def bench_recorded_4096(ct, O, dev, steps, warmup, check, nsets=4):
         ct.block_scaled_matmul(a_q, a_sw, b_q.T, b_sw, C=c, cache_scales=True)
 
     t_call_cached = _time_events(step_cached, steps, max(warmup, 2 * nsets))
-    packed = [(s[0], ct.pack_scales(s[1]), s[2].T, ct.pack_scales(s[3]), s[6]) for s in sets]
+    packed = [(s[0], ct.pack_scales(s[1], operand="a"), s[2].T, ct.pack_scales(s[3], operand="b"), s[6]) for s in sets]
     w = measure(lambda k: [t * 1e3 for t in ct.bench_block_scaled_matmul(packed, warmup=3, iters=k)], batch=10)
     flops = 2.0 * M * N * K
     return {"call_us_incl_scale_relayout": t_call * 1e6, "tflops": flops / t_call * 1e-12,
@@ -375,7 +376,7 @@ def bench_moe(ct, O, dev, steps, warmup, check, full_forward=True):
         ct.invoke_fused_moe_scaled(x_q, x_s, W, Ws, C, None, sid, eid, False, topk, tile)
 
     t_step = _time_wall(step, steps, warmup)
-    pW = ct.pack_scales(Ws)
+    pW = ct.pack_scales(Ws, operand="b")
 
     def kernel_mostly(i):
         ct.invoke_fused_moe_scaled(x_q, x_s, W, pW, C, None, sid, eid, False, topk, tile)

@@ -41,6 +41,13 @@ inline bool big_tile_problem(int64_t M, int64_t N) {
   return M > 128 && N > 128 && ((M + 255) / 256) * ((N + 255) / 256) >= 144;
 }
 
+// native scale layout a kernel reads: the two kernels on the 32x32x64 instruction have their own
+inline int native_layout_of(int kernel) {
+  return (kernel == MX_KERNEL_MFMA_PINGPONG32 || kernel == MX_KERNEL_MFMA_W4_PERSISTENT) ? MX_SCALE_NATIVE32
+                                                                                       : MX_SCALE_NATIVE;
+}
+inline bool is_native(int layout) { return layout == MX_SCALE_NATIVE || layout == MX_SCALE_NATIVE32; }
+
 const mx_gemm_opts kDefaultOpts = {sizeof(mx_gemm_opts), 0, MX_SCALE_2D, MX_SCALE_2D, MX_KERNEL_AUTO, 32, 0, 0};
 
 // Number of K-slices for a problem that ends up on a one-tile MFMA kernel (1 = no split).  Depends only on
@@ -153,8 +160,8 @@ int64_t mx_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, const mx_gemm_o
     b += round256(S * M * N * 4);
     return b;
   }
-  if (o.a_scale_layout != MX_SCALE_NATIVE) b += mx_packed_scale_bytes(M, K);
-  if (o.b_scale_layout != MX_SCALE_NATIVE) b += mx_packed_scale_bytes(N, K);
+  if (!is_native(o.a_scale_layout)) b += mx_packed_scale_bytes(M, K);
+  if (!is_native(o.b_scale_layout)) b += mx_packed_scale_bytes(N, K);
   return b;
 }
 
@@ -163,7 +170,7 @@ int64_t mx_gemm_grouped_workspace_bytes(int64_t num_slots, int64_t N, int64_t K,
   const mx_gemm_opts& o = opts ? *opts : kDefaultOpts;
   if (o.kernel == MX_KERNEL_GENERIC) return 0;
   int64_t b = mx_packed_scale_bytes(num_slots, K);
-  if (o.b_scale_layout != MX_SCALE_NATIVE) b += E * mx_packed_scale_bytes(N, K);
+  if (!is_native(o.b_scale_layout)) b += E * mx_packed_scale_bytes(N, K);
   return b;
 }
 
@@ -182,7 +189,8 @@ int check_swizzled_scale(const mx_tensor* scale, const char* name, int64_t rows,
 }
 
 // validates a scale tensor against (rows, K) and describes its re-layout into `packed`
-int make_pack_args(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, void* packed, PackArgs& p) {
+int make_pack_args(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, void* packed, int target,
+                   PackArgs& p) {
   if (int rc = check_tensor(scale, "scale", 2, 4)) return rc;
   if (!packed) return set_error(MX_ERR_INVALID, "packed: null pointer");
   if (K % 32 != 0) return set_error(MX_ERR_SHAPE, "K (%lld) must be a multiple of 32", (long long)K);
@@ -193,6 +201,7 @@ int make_pack_args(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t
   p.rows = rows;
   p.K = K;
   p.layout = layout;
+  p.target = target;
   p.batch = 1;
   p.replicas = 1;
   const int64_t KB = K / 32;
@@ -218,10 +227,15 @@ int make_pack_args(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t
 }
 }  // namespace
 
-int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, void* packed,
-                   void* stream) {
+int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, int32_t native_layout,
+                   int32_t operand, void* packed, void* stream) {
+  if (!is_native(native_layout))
+    return set_error(MX_ERR_INVALID, "mx_pack_scales: native_layout must be MX_SCALE_NATIVE or MX_SCALE_NATIVE32");
+  if (operand != MX_OPERAND_A && operand != MX_OPERAND_B)
+    return set_error(MX_ERR_INVALID, "mx_pack_scales: operand must be MX_OPERAND_A or MX_OPERAND_B");
+  const int target = native_layout == MX_SCALE_NATIVE32 ? kPackTile32 : (operand == MX_OPERAND_B ? kPackB : kPackA);
   PackArgs p;
-  if (int rc = make_pack_args(scale, layout, rows, K, packed, p)) return rc;
+  if (int rc = make_pack_args(scale, layout, rows, K, packed, target, p)) return rc;
   return launch_pack_scales(p, (hipStream_t)stream);
 }
 
@@ -362,7 +376,7 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
                      o.split_k, kernel);
   if (plan && kernel != MX_KERNEL_MFMA_128x128) return kPlanNotSimple;
   if (kernel == MX_KERNEL_GENERIC) {
-    if (o.a_scale_layout == MX_SCALE_NATIVE || o.b_scale_layout == MX_SCALE_NATIVE)
+    if (is_native(o.a_scale_layout) || is_native(o.b_scale_layout))
       return set_error(MX_ERR_LAYOUT, "the generic kernel cannot read native-layout scales");
     if (As->dtype == MX_E4M3 && !(A->dtype == MX_E2M1 && o.block_size == 16))
       return set_error(MX_ERR_DTYPE, "E4M3 scales are only defined for FP4 operands with block size 16");
@@ -442,14 +456,14 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
   if (S > 1) {
     // ---- split-K: the slices are a batch for the scale re-layout and a second grid dimension for the GEMM
     const int64_t Ks = K / S, kbs = Ks / 32;
-    if (int rc = make_pack_args(As, MX_SCALE_2D, M, K, ws, pa)) return rc;
+    if (int rc = make_pack_args(As, MX_SCALE_2D, M, K, ws, kPackA, pa)) return rc;
     pa.K = Ks; pa.batch = S; pa.s_batch = kbs * pa.s_kb;
     const uint32_t* as_p = (const uint32_t*)ws;
     ws += S * mx_packed_scale_bytes(M, Ks);
     mx_tensor t = *Bs;   // [K/32, N] -> view as [N, K/32]
     t.shape[0] = Bs->shape[1]; t.shape[1] = Bs->shape[0];
     t.stride[0] = Bs->stride[1]; t.stride[1] = Bs->stride[0];
-    if (int rc = make_pack_args(&t, MX_SCALE_2D, N, K, ws, pb)) return rc;
+    if (int rc = make_pack_args(&t, MX_SCALE_2D, N, K, ws, kPackB, pb)) return rc;
     pb.K = Ks; pb.batch = S; pb.s_batch = kbs * pb.s_kb;
     const uint32_t* bs_p = (const uint32_t*)ws;
     ws += S * mx_packed_scale_bytes(N, Ks);
@@ -469,9 +483,16 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
     if (int rc = launch_gemm_mfma(g, kernel, (hipStream_t)stream)) return rc;
     return launch_splitk_reduce(partial, S, M, N, C->ptr, C->stride[0], C->dtype, o.accumulate, (hipStream_t)stream);
   }
-  const bool pack_a = o.a_scale_layout != MX_SCALE_NATIVE, pack_b = o.b_scale_layout != MX_SCALE_NATIVE;
+  // (the decode and general kernels returned above: from here on `kernel` is one that reads a native layout)
+  const int native = native_layout_of(kernel);
+  const bool pack_a = !is_native(o.a_scale_layout), pack_b = !is_native(o.b_scale_layout);
+  if ((!pack_a && o.a_scale_layout != native) || (!pack_b && o.b_scale_layout != native))
+    return set_error(MX_ERR_LAYOUT, "kernel %d reads native-layout scales of kind %d (MX_SCALE_NATIVE for the "
+                     "16x16x128-instruction kernels, MX_SCALE_NATIVE32 for pingpong32 / w4p); pass the matching "
+                     "layout or the plain 2-D scales", kernel, native);
+  const bool t32 = native == MX_SCALE_NATIVE32;
   if (pack_a) {
-    if (int rc = make_pack_args(As, o.a_scale_layout, M, K, ws, pa)) return rc;
+    if (int rc = make_pack_args(As, o.a_scale_layout, M, K, ws, t32 ? kPackTile32 : kPackA, pa)) return rc;
     as_native = (const uint32_t*)ws;
     ws += mx_packed_scale_bytes(M, K);
   }
@@ -481,7 +502,7 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
       t.shape[0] = Bs->shape[1]; t.shape[1] = Bs->shape[0];
       t.stride[0] = Bs->stride[1]; t.stride[1] = Bs->stride[0];
     }
-    if (int rc = make_pack_args(&t, o.b_scale_layout, N, K, ws, pb)) return rc;
+    if (int rc = make_pack_args(&t, o.b_scale_layout, N, K, ws, t32 ? kPackTile32 : kPackB, pb)) return rc;
     bs_native = (const uint32_t*)ws;
   }
   if (((uintptr_t)as_native) % 16 != 0 || ((uintptr_t)bs_native) % 16 != 0)
@@ -684,7 +705,7 @@ int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W,
   if (K % 32 != 0) return set_error(MX_ERR_SHAPE, "K (%lld) must be a multiple of 32", (long long)K);
   const int64_t KB = K / 32;
   if (As->shape[0] != T || As->shape[1] != KB) return set_error(MX_ERR_SHAPE, "A_scale must be [tokens, K/32]");
-  if (o.b_scale_layout != MX_SCALE_NATIVE && (Ws->shape[0] != E || Ws->shape[1] != N || Ws->shape[2] != KB))
+  if (!is_native(o.b_scale_layout) && (Ws->shape[0] != E || Ws->shape[1] != N || Ws->shape[2] != KB))
     return set_error(MX_ERR_SHAPE, "W_scale must be [experts, N, K/32]");
   if (C->shape[1] != N || C->shape[0] < num_valid_ids)
     return set_error(MX_ERR_SHAPE, "C must be [>= num_valid_ids, N]");
@@ -742,7 +763,10 @@ int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W,
                      (long long)workspace_bytes);
   if (((uintptr_t)ws) % 256 != 0) return set_error(MX_ERR_WORKSPACE, "workspace must be 256-byte aligned");
   // A scales: gathered into slot order while re-laying; W scales of all experts ride in the same launch
+  const int native = native_layout_of(kernel);
+  const bool t32 = native == MX_SCALE_NATIVE32;
   PackArgs pa = {}, pw;
+  pa.target = t32 ? kPackTile32 : kPackA;
   pa.src = (const uint8_t*)As->ptr; pa.dst = (uint32_t*)ws;
   pa.rows = num_slots; pa.K = K; pa.s_row = As->stride[0]; pa.s_kb = As->stride[1];
   pa.layout = MX_SCALE_2D; pa.batch = 1;
@@ -750,10 +774,15 @@ int mx_gemm_grouped(const mx_tensor* A, const mx_tensor* As, const mx_tensor* W,
   const uint32_t* as_native = (const uint32_t*)ws;
   ws += mx_packed_scale_bytes(num_slots, K);
   const uint32_t* bs_native = (const uint32_t*)Ws->ptr;
-  const bool pack_w = o.b_scale_layout != MX_SCALE_NATIVE;
+  const bool pack_w = !is_native(o.b_scale_layout);
+  if (!pack_w && o.b_scale_layout != native)
+    return set_error(MX_ERR_LAYOUT, "kernel %d reads native-layout scales of kind %d, W_scale has kind %d", kernel,
+                     native, o.b_scale_layout);
+  if (E * mx_packed_scale_bytes(N, K) >= ((int64_t)1 << 31))
+    return set_error(MX_ERR_SHAPE, "the packed scales of all experts must stay below 2 GiB");
   if (pack_w) {
     if (o.b_scale_layout != MX_SCALE_2D) return set_error(MX_ERR_LAYOUT, "W_scale must be [E, N, K/32] or native");
-    if (int rc = make_pack_args(Ws, MX_SCALE_2D, N, K, ws, pw)) return rc;
+    if (int rc = make_pack_args(Ws, MX_SCALE_2D, N, K, ws, t32 ? kPackTile32 : kPackB, pw)) return rc;
     bs_native = (const uint32_t*)ws;
   }
   if (int rc = launch_pack_scales_pair(&pa, pack_w ? &pw : nullptr, (hipStream_t)stream)) return rc;

@@ -385,6 +385,7 @@ constexpr int kPackListMax = 64;
 struct PackEntry {
   const uint8_t* src; uint32_t* dst;
   int64_t rows, K, s_row, s_kb;
+  int32_t target;
 };
 struct PackList {
   PackEntry p[kPackListMax];
@@ -441,14 +442,24 @@ __device__ inline void pack_scales_block(const PackArgs& p, const int64_t blk) {
   }
   __syncthreads();
 
-  // ---- assemble: thread = (quad q of the group, lane); dword i4 = row 16 i4 + lane % 16, byte t =
-  // K block (4 (Q0 + q) + t) * 4 + lane / 16 -----------------------------------------------------------------
+  // ---- assemble: thread = (quad q of the group, lane): the 4 x 4 bytes (row, K-step) of the lane, K block
+  // (4 (Q0 + q) + t) * 4 + lane / 16 for K-step t; which rows and which index is the dword depend on the target ---
   const int q = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
   if (Q0 + q >= KQ) return;
   uint32_t out[4];
-  for (int i4 = 0; i4 < 4; ++i4) {
-    const uint8_t* t = tile + (i4 * 16 + r) * LD + q * 16 + g;
-    out[i4] = (uint32_t)t[0] | ((uint32_t)t[4] << 8) | ((uint32_t)t[8] << 16) | ((uint32_t)t[12] << 24);
+  if (p.target == kPackTile32) {
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const uint8_t* t = tile + (i4 * 16 + r) * LD + q * 16 + g;
+      out[i4] = (uint32_t)t[0] | ((uint32_t)t[4] << 8) | ((uint32_t)t[8] << 16) | ((uint32_t)t[12] << 24);
+    }
+  } else {
+    int row[4];
+    for (int b = 0; b < 4; ++b) row[b] = p.target == kPackB ? bperm_row(b, r) : 16 * b + r;
+    for (int t = 0; t < 4; ++t) {
+      const uint8_t* c = tile + q * 16 + 4 * t + g;
+      out[t] = (uint32_t)c[row[0] * LD] | ((uint32_t)c[row[1] * LD] << 8) | ((uint32_t)c[row[2] * LD] << 16) |
+               ((uint32_t)c[row[3] * LD] << 24);
+    }
   }
   uint32_t* dst = p.dst + b * packed_scale_dwords(p.rows, p.K) + ((t64 * KQ + Q0 + q) * 64 + lane) * 4;
   *(uint4*)dst = make_uint4(out[0], out[1], out[2], out[3]);
@@ -465,6 +476,7 @@ __global__ __launch_bounds__(256) void pack_scales_list_kernel(const PackList pl
   const PackEntry& e = pl.p[i];
   PackArgs p = {};
   p.src = e.src; p.dst = e.dst; p.rows = e.rows; p.K = e.K; p.s_row = e.s_row; p.s_kb = e.s_kb;
+  p.target = e.target;
   p.layout = MX_SCALE_2D; p.batch = 1; p.replicas = 1;
   pack_scales_block(p, (int)blockIdx.x - pl.first_block[i]);
 }
@@ -718,7 +730,7 @@ int launch_pack_scales_list(const PackArgs* list, int n, hipStream_t stream) {
       if (p.rows <= 0 || p.K <= 0 || p.batch <= 0) continue;
       if (p.layout != MX_SCALE_2D || p.batch != 1 || p.gather_ids)
         return set_error(MX_ERR_INVALID, "pack_scales list: plain 2-D scale tensors only");
-      pl.p[pl.n] = PackEntry{p.src, p.dst, p.rows, p.K, p.s_row, p.s_kb};
+      pl.p[pl.n] = PackEntry{p.src, p.dst, p.rows, p.K, p.s_row, p.s_kb, p.target};
       pl.first_block[pl.n] = (int32_t)total;
       total += ((p.rows + 63) / 64) * ((packed_scale_quads(p.K) + 3) / 4) * p.batch;
       if (total > 0x7FFFFFFF) return set_error(MX_ERR_SHAPE, "pack_scales: tensors too large");

@@ -16,12 +16,29 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 // ---- error reporting (host) ------------------------------------------------------------------
 int set_error(int code, const char* fmt, ...);
 
-// ---- native scale layout -----------------------------------------------------------------------
-// One dword per (16-row tile I, K-quad Q, lane): byte t (0..3) is the E8M0 scale of row
-// 16*I + lane%16 for the 32-element K block  (4*Q + t)*4 + lane/16, i.e. MFMA K-step 4*Q + t
-// (128 elements) and lane group lane/16.  Dwords are stored as [I/4][Q][lane][I%4] so that one
-// 16-byte load per lane brings the scales of four row tiles for four K-steps.
-// Rows are padded to a multiple of 64 and K-steps to a multiple of 4 with the byte 127 (1.0).
+// ---- native scale layouts ----------------------------------------------------------------------
+// Both hold 16 bytes per (64-row group G, K-quad Q of four 128-element MFMA K-steps, lane), stored [G][Q][lane]:
+// a 4 x 4 byte matrix of the scales of four rows for the four K-steps of the quad, for the 32-element K block
+// (4 Q + t) * 4 + lane / 16 of K-step t.  One 16-byte load per lane (1 KiB contiguous per wave) brings a group's
+// scales for a quad.  Rows are padded to a multiple of 64 and K-steps to a multiple of 4 with the byte 127 (1.0).
+//   MX_SCALE_NATIVE (kernels on the 16x16x128 instruction): dword t = K-step, byte b = row, so that one register
+//     feeds the four 16-row tiles of a group for one K-step (the tile is picked by the instruction's byte select).
+//       A operand (kPackA): byte b = row 64 G + 16 b + lane % 16
+//       B operand (kPackB): byte b = row 64 G + bperm_row(b, lane % 16), the row order in which the kernels feed
+//                           B to the instruction
+//   MX_SCALE_NATIVE32 (kernels on the 32x32x64 instruction, kPackTile32): dword b = row 64 G + 16 b + lane % 16,
+//     byte t = K-step; both operands alike.
+enum { kPackA = 0, kPackB = 1, kPackTile32 = 2 };
+// ---- column order of the 16x16x128 kernels' B fragments ------------------------------------------------
+// MFMA tile j (0..3) of a wave's 64 B rows takes, as its operand row c, B row
+//     bperm_row(j, c) = 32 (j / 2) + 8 (c / 4) + 4 (j % 2) + c % 4
+// instead of 16 j + c.  Lane (c, g) of the result then holds columns 32 (j / 2) + 8 g + 4 (j % 2) + e,
+// e = 0..3: the tiles j = 2p and 2p + 1 give it 8 consecutive outputs, which leave as one 16-byte (bf16) or
+// two adjacent 16-byte (fp32) stores -- half as many store instructions as with 4 consecutive outputs.
+__host__ __device__ inline int bperm_tile_off(int j) { return 32 * (j >> 1) + 4 * (j & 1); }   // part of the row that depends on j
+__host__ __device__ inline int bperm_lane_off(int c) { return 8 * (c >> 2) + (c & 3); }         // part that depends on the lane
+__host__ __device__ inline int bperm_row(int j, int c) { return bperm_tile_off(j) + bperm_lane_off(c); }
+
 __host__ __device__ inline int64_t packed_scale_quads(int64_t K) { return (K + 511) / 512; }
 __host__ __device__ inline int64_t packed_scale_dwords(int64_t rows, int64_t K) {
   return ((rows + 63) / 64) * packed_scale_quads(K) * 256;
@@ -143,6 +160,7 @@ struct PackArgs {
   int64_t s_batch, s_row, s_kb;  // byte strides of the 2-D source
   int32_t layout;                // MX_SCALE_2D / MX_SCALE_SWIZZLE_32_4_4
   int32_t batch;
+  int32_t target;                // kPackA / kPackB / kPackTile32
   // optional row gather (grouped GEMM): row p reads source row idx[p] / replicas if idx[p] < num_valid
   const int32_t* gather_ids; int32_t replicas; int64_t num_valid_ids;
 };

@@ -103,7 +103,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, lds_u8* const smem,
   for (int q = 0; q < C::B_LOADS; ++q) {
     const int slot = (q * C::NW + wave) * 64 + lane;
     const int row = slot / C::B_CPR, pos = slot % C::B_CPR;
-    const int col = (pos ^ swz<C::B_CPR>(row)) * 16;
+    const int col = (pos ^ swz_bperm<C::B_CPR>(row)) * 16;   // the swizzle of the permuted fragment reads below
     b_col[q] = col;
     int64_t grow = n0 + row;
     b_voff[q] = grow < g.N ? (uint32_t)(grow * g.ldb + col) : kOobOffset;
@@ -130,7 +130,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, lds_u8* const smem,
     }
   };
 
-  // ---- scales: one 16-byte load per lane covers 4 row tiles x 4 K-steps ------------------------------
+  // ---- scales: one 16-byte load per lane covers 4 row tiles x 4 K-steps (dword = K-step, byte = tile) ---
   constexpr int AQ = C::MT / 4, BQ = C::NTL / 4;
   // the packed tensors hold ceil(rows / 64) row groups; a tile that hangs over the matrix edge re-reads
   // the last group (its rows are never stored)
@@ -193,28 +193,23 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, lds_u8* const smem,
         const bool more = it + 1 < nstages;
         const int sn = (t0 / C::KSUB + 1 < SPQ) ? s + 1 : Qn * SPQ;   // stage that follows in the walk
         lds_u8* const atile = smem + buf * C::STAGE + (wm0 + r) * C::A_RB;
-        lds_u8* const btile = smem + buf * C::STAGE + C::A_STAGE + (wn0 + r) * C::B_RB;
+        // B rows go to the instruction in the order bperm_row (mx_common.h): tile j of a 64-row group is rows
+        // bperm_tile_off(j) + bperm_lane_off(lane % 16), which is also the order of the packed B scales
+        lds_u8* const btile = smem + buf * C::STAGE + C::A_STAGE + (wn0 + bperm_lane_off(r)) * C::B_RB;
 #pragma unroll
         for (int kk = 0; kk < C::KSUB; ++kk) {
           v8i bf[C::NTL];
 #pragma unroll
           for (int j = 0; j < C::NTL; ++j) {
-            bf[j] = load_frag<C::B_RB, C::B_EB>(btile, 16 * j, kk, gq, swb);
+            bf[j] = load_frag<C::B_RB, C::B_EB>(btile, 64 * (j / 4) + bperm_tile_off(j % 4), kk, gq, swb);
           }
 #pragma unroll
           for (int i = 0; i < C::MT; ++i) {
             const v8i af = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
 #pragma unroll
             for (int j = 0; j < C::NTL; ++j) {
-              // compile-time K-step index within the quad selects the scale byte
-              if (t0 + kk == 0)
-                acc[i][j] = mfma_scaled<C::BF, C::AF, 0>(bf[j], af, acc[i][j], sb[j / 4][j % 4], sa[i / 4][i % 4]);
-              else if (t0 + kk == 1)
-                acc[i][j] = mfma_scaled<C::BF, C::AF, 1>(bf[j], af, acc[i][j], sb[j / 4][j % 4], sa[i / 4][i % 4]);
-              else if (t0 + kk == 2)
-                acc[i][j] = mfma_scaled<C::BF, C::AF, 2>(bf[j], af, acc[i][j], sb[j / 4][j % 4], sa[i / 4][i % 4]);
-              else
-                acc[i][j] = mfma_scaled<C::BF, C::AF, 3>(bf[j], af, acc[i][j], sb[j / 4][j % 4], sa[i / 4][i % 4]);
+              acc[i][j] = mfma_scaled<C::BF, C::AF>(bf[j], af, acc[i][j], j % 4, sb[j / 4][t0 + kk], i % 4,
+                                                    sa[i / 4][t0 + kk]);
             }
             if (kk == 0 && i < LOAD_ITERS) {
 #pragma unroll
@@ -234,7 +229,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, lds_u8* const smem,
     for (int u = 0; u < BQ; ++u) sb[u] = sb_n[u];
   }
 
-  // ---- epilogue: lane (r, gq) of tile (i, j) holds C[m0+wm0+16i+r][n0+wn0+16j+4gq .. +3] -----------
+  // ---- epilogue: lane (r, gq) of tile (i, j) holds row m0 + wm0 + 16 i + r, columns
+  // n0 + wn0 + 64 (j / 4) + bperm_tile_off(j % 4) + 8 gq .. + 3 -----------------------------------------------
   OutT* const Cp = (OutT*)g.C + (int64_t)split * g.c_split_stride;
   const bool vec_ok = (g.ldc % 4 == 0) && (((uintptr_t)g.C) % 16 == 0) && (g.c_split_stride % 4 == 0);
   const bool accumulate = g.accumulate != 0;
@@ -253,7 +249,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, lds_u8* const smem,
     if (!ok) continue;
 #pragma unroll
     for (int j = 0; j < C::NTL; ++j) {
-      const int n = n0 + wn0 + 16 * j + 4 * gq;
+      const int n = n0 + wn0 + 64 * (j / 4) + bperm_tile_off(j % 4) + 8 * gq;
       if (n >= g.N) continue;
       v4f v = acc[i][j];
       if constexpr (GROUPED) v *= w;

@@ -18,7 +18,6 @@ struct PP {
   static constexpr int A_RPI = 64 / C::A_CPR, B_RPI = 64 / C::B_CPR;   // rows per DMA instruction
   static constexpr int AL = 128 / A_RPI / 4;                // A loads per wave and stage
   static constexpr int BL = 64 / B_RPI;                     // B loads per team-1 wave and stage
-  static constexpr int SCALE_LOADS = 6;                     // two A groups (16 bytes each), four B tiles (4 bytes each)
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 

@@ -95,18 +95,23 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
   // swizzled byte column of DMA instruction q (rows b_row0 + q * B_RPI ...)
   auto b_col = [&](int q) { return ((lane % C::B_CPR) ^ swz_bperm<C::B_CPR>(lane / C::B_CPR + q * P::B_RPI)) * 16; };
   __amdgpu_buffer_rsrc_t rsB;
-  // scale groups (16-byte index of K-quad 0, lane 0) of this wave's rows / columns: for the tile being
-  // computed and for the tile being fetched
+  // ---- scales (native layout, mx_common.h): 16 bytes per (64-row group, K-quad, lane), dword t = K-step t of the
+  // quad, byte = 16-row tile of the group (B: in the bperm_row order of the fragments).  A K-quad needs the team's
+  // two A groups and the wave's one B group: three 16-byte loads (1 KiB contiguous per wave) through buffer
+  // descriptors, the (group, quad) part of the address in the scalar offset.
+  // as / bs _cur, _nxt: byte offset of (group, K-quad 0) for the tile being computed / being fetched.
   int as_cur[2], bs_cur, as_nxt[2], bs_nxt;
-  v4i sb;   // scale dwords of the wave's four B tiles for the current K-quad
-  const v4i* const As4 = (const v4i*)g.As + lane;
-  // B scales: tile j of this lane is B row bperm_row(j, r) = 16-row group 2 (j / 2) + r / 8 of the wave's 64 rows,
-  // row 8 (r / 4 % 2) + 4 (j % 2) + r % 4 inside it; in the packed layout ([64-row group][K-quad][lane][group % 4]
-  // dwords, lane = row % 16 + 16 * K-block) that is one dword per tile, 16 (j % 2) + 2 (j / 2) dwords apart
-  const int* const Bs1 = (const int*)g.Bs + 4 * (8 * ((r >> 2) & 1) + (r & 3) + 16 * gq) + (r >> 3);
-  auto load_b_scales = [&](int idx16) {   // idx16: 16-byte index of (64-row group, K-quad), lane 0
+  const __amdgpu_buffer_rsrc_t rsAs = make_rsrc(g.As, (uint32_t)(packed_scale_dwords(g.M, g.K) * 4));
+  const __amdgpu_buffer_rsrc_t rsBs =
+      make_rsrc(g.Bs, (uint32_t)((GROUPED ? (int64_t)(g.num_experts - 1) * g.bs_expert_stride * 4 : 0) +
+                                 packed_scale_dwords(g.N, g.K) * 4));
+  const int sc_voff = lane * 16;
+  constexpr int NSC = 3;           // scale load instructions per K-quad
+  v4i sa[2], sb;
+  auto load_scales = [&](const int* as_off, int bs_off, int Qn) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) sb[j] = Bs1[(int64_t)idx16 * 4 + 16 * (j & 1) + 2 * (j >> 1)];
+    for (int u = 0; u < 2; ++u) sa[u] = __builtin_amdgcn_raw_buffer_load_b128(rsAs, sc_voff, as_off[u] + Qn * 1024, 0);
+    sb = __builtin_amdgcn_raw_buffer_load_b128(rsBs, sc_voff, bs_off + Qn * 1024, 0);
   };
   bool fetch_valid = true;   // false once the walk has no further tile: loads become zero-fill no-ops
   // grouped: none of this team's 128 slots of the tile holds a routed row (every slot is looked at: two per lane,
@@ -161,11 +166,11 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int grp = (m0 + wm0) / 64 + u;
-      as_nxt[u] = (grp < a_groups ? grp : a_groups - 1) * KQ * 64;
+      as_nxt[u] = (grp < a_groups ? grp : a_groups - 1) * KQ * 1024;
     }
     const int grp = (n0 + wn0) / 64;
-    bs_nxt = (GROUPED ? (int)(expert * (g.bs_expert_stride / 4)) : 0) +
-             (grp < b_groups ? grp : b_groups - 1) * KQ * 64;
+    bs_nxt = (GROUPED ? (int)(expert * (g.bs_expert_stride * 4)) : 0) +
+             (grp < b_groups ? grp : b_groups - 1) * KQ * 1024;
   };
   // local stage sl of the fetch tile into A buffer abuf / B buffer bbuf; a stage at or beyond nstages
   // and the 16-byte chunks beyond the end of K read nothing and zero-fill their LDS bytes
@@ -196,7 +201,6 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     }
   };
 
-  v4i sa[2];
   v4f acc[8][4];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
@@ -313,12 +317,10 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     // =============================== memory phase ==================================================
     if constexpr (t0 == 0) {
       // Scales of this K-quad, first in the queue of this memory phase: they have the whole phase to arrive, and
-      // the MFMA phase holds no vector-memory instruction at all.  (Issued at the end of the previous quad's last
-      // MFMA phase instead, they met the other team's DMA burst in the address unit and held this team's arrival
-      // at the barrier: 2 % slower on MXFP8, 1 % on MXFP4.)
-#pragma unroll
-      for (int u = 0; u < 2; ++u) sa[u] = As4[as_cur[u] + Q * 64];
-      load_b_scales(bs_cur + Q * 64);
+      // the MFMA phase holds no vector-memory instruction at all.  (Requested a stage ahead, stage by stage, in
+      // 4-byte loads, they arrive no earlier in effect: what they cost is their share of the address unit, which
+      // three 16-byte loads per quad keep smallest.)
+      load_scales(as_cur, bs_cur, Q);
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (t0 == 0) {
@@ -362,7 +364,7 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       issue_b(sl_eff, bbuf);
       // everything older than this phase's loads has landed: A and B of stage s + 1 (the scale loads issued
       // at the start of this phase are younger than those and may stay in flight; the MFMA phase waits for them)
-      constexpr int younger = (t0 == 0) ? P::SCALE_LOADS : 0;
+      constexpr int younger = (t0 == 0) ? NSC : 0;
       __builtin_amdgcn_s_waitcnt(vmcnt_imm(AL + BL + younger));
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -386,14 +388,8 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
         for (int i = i0; i < i0 + 2; ++i) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            if (t0 + kk == 0)
-              acc[i][j] = mfma_scaled<C::BF, C::AF, 0>(bf[kk][j], af[kk][i], acc[i][j], sb[j], sa[i / 4][i % 4]);
-            else if (t0 + kk == 1)
-              acc[i][j] = mfma_scaled<C::BF, C::AF, 1>(bf[kk][j], af[kk][i], acc[i][j], sb[j], sa[i / 4][i % 4]);
-            else if (t0 + kk == 2)
-              acc[i][j] = mfma_scaled<C::BF, C::AF, 2>(bf[kk][j], af[kk][i], acc[i][j], sb[j], sa[i / 4][i % 4]);
-            else
-              acc[i][j] = mfma_scaled<C::BF, C::AF, 3>(bf[kk][j], af[kk][i], acc[i][j], sb[j], sa[i / 4][i % 4]);
+            acc[i][j] = mfma_scaled<C::BF, C::AF>(bf[kk][j], af[kk][i], acc[i][j], j, sb[t0 + kk], i % 4,
+                                                  sa[i / 4][t0 + kk]);
           }
         }
       }

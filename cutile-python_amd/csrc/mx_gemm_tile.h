@@ -42,14 +42,6 @@ __device__ inline int swz(int row) {
   return (row / (16 / CPR)) % CPR;
 }
 
-// ---- column order of the ping-pong kernel's B fragments ------------------------------------------------
-// MFMA tile j (0..3) of a wave's 64 B rows takes, as its operand row c, B row
-//     bperm_row(j, c) = 32 (j / 2) + 8 (c / 4) + 4 (j % 2) + c % 4
-// instead of 16 j + c.  Lane (c, g) of the result then holds columns 32 (j / 2) + 8 g + 4 (j % 2) + e,
-// e = 0..3: the tiles j = 2p and 2p + 1 give it 8 consecutive outputs, which leave as one 16-byte (bf16) or
-// two adjacent 16-byte (fp32) stores -- half as many store instructions as with 4 consecutive outputs.
-__device__ inline int bperm_tile_off(int j) { return 32 * (j >> 1) + 4 * (j & 1); }   // part of the row that depends on j
-__device__ inline int bperm_lane_off(int c) { return 8 * (c >> 2) + (c & 3); }         // part that depends on the lane
 // LDS swizzle of the B rows for that read pattern: built from the row bits that tell the 16 lanes of a read
 // apart beyond the bank half (CPR = 8: bits 1, 3, 4; CPR = 4: bits 3, 4); for row bperm_row(j, c) it equals
 // swz<CPR>(c), whatever j is.
@@ -75,11 +67,23 @@ __device__ inline v8i load_frag(lds_u8* tile, int row, int kk, int gq, int sw) {
   }
 }
 
-template <int BFMT, int AFMT, int T>
-__device__ inline v4f mfma_scaled(const v8i& bfrag, const v8i& afrag, const v4f& acc, int bscale,
-                                  int ascale) {
-  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bfrag, afrag, acc, BFMT, AFMT, T, bscale,
-                                                          T, ascale);
+// One scaled MFMA; the B fragment's scales are byte `bsel` of bscale, the A fragment's byte `asel` of ascale (in the
+// native scale layout a register holds one K-step's scales of four 16-row tiles, so the byte is the tile's index in
+// its group of four).  bsel and asel must fold to constants: the instruction encodes them.
+template <int BFMT, int AFMT>
+__device__ __forceinline__ v4f mfma_scaled(const v8i& bfrag, const v8i& afrag, const v4f& acc, int bsel, int bscale,
+                                           int asel, int ascale) {
+#define MX_MFMA_CASE(SB, SA)                                                                                   \
+  case SB * 4 + SA:                                                                                            \
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bfrag, afrag, acc, BFMT, AFMT, SB, bscale, SA, ascale);
+  switch (bsel * 4 + asel) {
+    MX_MFMA_CASE(0, 0) MX_MFMA_CASE(0, 1) MX_MFMA_CASE(0, 2) MX_MFMA_CASE(0, 3)
+    MX_MFMA_CASE(1, 0) MX_MFMA_CASE(1, 1) MX_MFMA_CASE(1, 2) MX_MFMA_CASE(1, 3)
+    MX_MFMA_CASE(2, 0) MX_MFMA_CASE(2, 1) MX_MFMA_CASE(2, 2) MX_MFMA_CASE(2, 3)
+    MX_MFMA_CASE(3, 0) MX_MFMA_CASE(3, 1) MX_MFMA_CASE(3, 2) MX_MFMA_CASE(3, 3)
+  }
+#undef MX_MFMA_CASE
+  __builtin_unreachable();
 }
 
 template <typename OutT>

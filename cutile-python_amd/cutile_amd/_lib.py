@@ -18,7 +18,10 @@ MX_ERR_WORKSPACE, MX_ERR_DEVICE, MX_ERR_LAUNCH = -5, -6, -7
 MX_E4M3, MX_E5M2, MX_E2M1, MX_E8M0 = 0, 1, 4, 8
 MX_F32, MX_BF16, MX_F16, MX_I32 = 16, 17, 18, 24
 
-MX_SCALE_2D, MX_SCALE_SWIZZLE_32_4_4, MX_SCALE_NATIVE = 0, 1, 2
+MX_SCALE_2D, MX_SCALE_SWIZZLE_32_4_4, MX_SCALE_NATIVE, MX_SCALE_NATIVE32 = 0, 1, 2, 3
+MX_OPERAND_A, MX_OPERAND_B = 0, 1
+# kernels that read MX_SCALE_NATIVE32 (the 32x32x64 instruction); every other MFMA kernel reads MX_SCALE_NATIVE
+NATIVE32_KERNELS = ("pingpong32", "w4p")
 
 MX_KERNEL_AUTO, MX_KERNEL_GENERIC = 0, 1
 MX_KERNEL_MFMA_128x128, MX_KERNEL_MFMA_256x256, MX_KERNEL_MFMA_256x256_W4, MX_KERNEL_DECODE = 2, 3, 4, 5
@@ -77,7 +80,7 @@ SYMBOLS = {
     "mx_silu_mul_quantize": (ctypes.c_int, [_P(MxTensor)] * 3 + [ctypes.c_int32, ctypes.c_void_p]),
     "mx_packed_scale_bytes": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int64]),
     "mx_pack_scales": (ctypes.c_int, [_P(MxTensor), ctypes.c_int32, ctypes.c_int64, ctypes.c_int64,
-                                      ctypes.c_void_p, ctypes.c_void_p]),
+                                      ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p]),
 }
 
 _lib = None

@@ -102,11 +102,15 @@ def _logical_shape(t: torch.Tensor, packed_dim: int) -> Tuple[int, ...]:
 
 @dataclass
 class PackedScales:
-    """Scales in the library's MFMA-ready layout (see :func:`pack_scales`)."""
+    """Scales in one of the library's MFMA-ready layouts (see :func:`pack_scales`): ``operand`` "a" or "b" says
+    which side of the product they were packed for, ``layout`` which kernels read them (``MX_SCALE_NATIVE``:
+    all MFMA kernels but "pingpong32" and "w4p", which read ``MX_SCALE_NATIVE32``)."""
     data: torch.Tensor   # uint8 [batch * bytes]
     rows: int
     K: int
     batch: int = 1
+    operand: str = "a"
+    layout: int = L.MX_SCALE_NATIVE
 
 
 def _as_u8(t: torch.Tensor) -> torch.Tensor:
@@ -133,6 +137,9 @@ def _scale_desc(s, rows: int, K: int, block: int, is_b: bool):
     if isinstance(s, PackedScales):
         if s.rows != rows or s.K != K:
             raise ValueError(f"packed scales were built for rows={s.rows}, K={s.K}; need rows={rows}, K={K}")
+        if s.operand != ("b" if is_b else "a"):
+            raise ValueError(f"scales packed for operand {s.operand!r} passed as operand {'b' if is_b else 'a'!r}: "
+                             "pack_scales(..., operand=...) orders the rows differently for the two sides")
         d = L.MxTensor()
         d.ptr = s.data.data_ptr()
         d.dtype = L.MX_E8M0
@@ -140,7 +147,7 @@ def _scale_desc(s, rows: int, K: int, block: int, is_b: bool):
         d.shape[0], d.shape[1] = rows, K // 32
         d.stride[0], d.stride[1] = K // 32, 1
         d.packed_dim = -1
-        return d, L.MX_SCALE_NATIVE
+        return d, s.layout
     code = _scale_code(s)
     if s.dim() == 4:
         return L.desc(_as_u8(s), code), L.MX_SCALE_SWIZZLE_32_4_4
@@ -178,7 +185,7 @@ class _ScaleCache:
                     # so that dropping the entry while this stream's GEMM is in flight does not recycle the block
                     e[2].data.record_stream(stream)
                 return e[2]
-        packed = pack_scales(s, transposed=transposed)
+        packed = pack_scales(s, transposed=transposed, operand="b" if transposed else "a")
         if torch.cuda.is_current_stream_capturing():
             return packed                             # memory of the capture's private pool: not for later eager calls
         ev = torch.cuda.Event()
@@ -617,13 +624,21 @@ def unswizzle_32_4_4(sw: torch.Tensor) -> torch.Tensor:
     return sw.reshape(m0, k0, m1, m2, k1).permute(0, 3, 2, 1, 4).reshape(m0 * m2 * m1, k0 * k1)
 
 
-def pack_scales(scale: torch.Tensor, *, transposed: bool = False) -> PackedScales:
+def pack_scales(scale: torch.Tensor, *, transposed: bool = False, operand: Optional[str] = None,
+                kernel: str = "auto") -> PackedScales:
     """Re-lays E8M0 scales once into the layout the MFMA kernels read directly, so repeated GEMMs with
     the same operand (weights) skip the per-call re-layout.  ``scale`` is [rows, K/32] (``transposed``:
     [K/32, rows], as B_scale is passed), optionally with a leading batch (experts) dimension, or the
-    4-D swizzle_32_4_4 tensor."""
+    4-D swizzle_32_4_4 tensor.  ``operand``: "a" for the left operand (activations), "b" for the right one
+    (weights, expert weights); the two are packed differently.  Default: "b" for a transposed or batched
+    tensor, else "a".  ``kernel``: the kernel the scales are for; only "pingpong32" and "w4p" differ from the rest."""
     if not scale.is_cuda:
         raise ValueError("Input tensors must be on a CUDA device.")
+    if operand is None:
+        operand = "b" if (transposed or scale.dim() == 3) else "a"
+    if operand not in ("a", "b"):
+        raise TileValueError(f"operand must be 'a' or 'b', got {operand!r}")
+    native = L.MX_SCALE_NATIVE32 if kernel in L.NATIVE32_KERNELS else L.MX_SCALE_NATIVE
     s = _as_u8(scale)
     lib = L.lib()
     if s.dim() == 4:
@@ -638,9 +653,11 @@ def pack_scales(scale: torch.Tensor, *, transposed: bool = False) -> PackedScale
     out = torch.empty(batch * nbytes, dtype=torch.uint8, device=s.device)
     d = L.desc(s, L.MX_E8M0)
     with torch.cuda.device(s.device):
-        rc = lib.mx_pack_scales(ctypes.byref(d), layout, rows, K, out.data_ptr(), L.stream_ptr(s.device))
+        rc = lib.mx_pack_scales(ctypes.byref(d), layout, rows, K, native,
+                                L.MX_OPERAND_B if operand == "b" else L.MX_OPERAND_A, out.data_ptr(),
+                                L.stream_ptr(s.device))
     _check(rc)
-    return PackedScales(out, rows, K, batch)
+    return PackedScales(out, rows, K, batch, operand, native)
 
 
 # ==================================================================================================
@@ -704,13 +721,15 @@ def invoke_fused_moe_scaled(A: torch.Tensor, A_scale: torch.Tensor, B: torch.Ten
     if isinstance(B_scale, PackedScales):
         if B_scale.rows != N or B_scale.K != K or B_scale.batch != E:
             raise ValueError("packed B_scale does not match B")
+        if B_scale.operand != "b":
+            raise ValueError("expert scales must be packed with operand='b'")
         dBs = L.MxTensor()
         dBs.ptr = B_scale.data.data_ptr()
         dBs.dtype, dBs.ndim = L.MX_E8M0, 3
         dBs.shape[0], dBs.shape[1], dBs.shape[2] = E, N, K // 32
         dBs.stride[0], dBs.stride[1], dBs.stride[2] = N * (K // 32), K // 32, 1
         dBs.packed_dim = -1
-        lb = L.MX_SCALE_NATIVE
+        lb = B_scale.layout
     else:
         dBs, lb = L.desc(_as_u8(B_scale), L.MX_E8M0), L.MX_SCALE_2D
     dC = L.desc(C2, L._TORCH_TO_MX[C2.dtype])

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MXGEMM_VERSION 102
+#define MXGEMM_VERSION 103
 
 /* Exported symbols (the library is built with hidden default visibility). */
 #if defined(__GNUC__)
@@ -85,7 +85,17 @@ enum {
   MX_SCALE_SWIZZLE_32_4_4 = 1, /* contiguous [rows/128, (K/B)/4, 32, 16] as produced by
                              swizzle_32_4_4 (test/kernels/kernel_utils.py:83-98); for B the rows
                              are the N index                                                      */
-  MX_SCALE_NATIVE = 2     /* this library's MFMA-ready layout written by mx_pack_scales          */
+  MX_SCALE_NATIVE = 2,    /* this library's MFMA-ready layout written by mx_pack_scales for the
+                             kernels on v_mfma_scale_f32_16x16x128_f8f6f4 (every MFMA kernel but the
+                             two below); A and B scales are packed differently (MX_OPERAND_*)      */
+  MX_SCALE_NATIVE32 = 3   /* the MFMA-ready layout of the kernels on v_mfma_scale_f32_32x32x64_f8f6f4
+                             (MX_KERNEL_MFMA_PINGPONG32, MX_KERNEL_MFMA_W4_PERSISTENT)             */
+};
+
+/* Which operand of the product a native-layout scale tensor belongs to (mx_pack_scales). */
+enum {
+  MX_OPERAND_A = 0,
+  MX_OPERAND_B = 1
 };
 
 /* Kernel selection. */
@@ -134,7 +144,7 @@ MX_API int mx_device_check(void);
 
 /*
  * Bytes of device workspace mx_gemm needs for the given problem (native re-layout of the scale
- * tensors).  0 if both scale tensors are already MX_SCALE_NATIVE or the generic kernel is used.
+ * tensors).  0 if both scale tensors are already in a native layout or the generic kernel is used.
  */
 MX_API int64_t mx_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, const mx_gemm_opts* opts);
 
@@ -278,16 +288,20 @@ MX_API int mx_silu_mul_quantize(const mx_tensor* gate_up, mx_tensor* xq, mx_tens
                          void* stream);
 
 /*
- * Re-lays a scale tensor into the MFMA-ready native layout consumed by the MFMA kernels
+ * Re-lays a scale tensor into an MFMA-ready native layout consumed by the MFMA kernels
  * (no reference counterpart: the reference's swizzle_32_4_4, test/kernels/kernel_utils.py:83-98,
  * is the Blackwell analogue).  `scale` is [rows, K/32] logical with any strides (MX_SCALE_2D; pass a
  * transposed descriptor for a [K/32, cols] tensor), or the contiguous 4-D swizzled tensor
  * (MX_SCALE_SWIZZLE_32_4_4); an optional leading batch dimension (experts) is kept.
- * `packed` must hold mx_packed_scale_bytes(rows, K) bytes per batch entry.
+ * `native_layout` is MX_SCALE_NATIVE or MX_SCALE_NATIVE32 (the kernels that will read it), `operand`
+ * MX_OPERAND_A (activations / left operand) or MX_OPERAND_B (weights / right operand, also the expert
+ * weights of mx_gemm_grouped): MX_SCALE_NATIVE orders the B rows the way the kernels feed them to the
+ * instruction, so a tensor packed for one operand must not be passed as the other.
+ * `packed` must hold mx_packed_scale_bytes(rows, K) bytes per batch entry (the same for every layout).
  */
 MX_API int64_t mx_packed_scale_bytes(int64_t rows, int64_t K);
-MX_API int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, void* packed,
-                   void* stream);
+MX_API int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, int32_t native_layout,
+                   int32_t operand, void* packed, void* stream);
 
 #ifdef __cplusplus
 }

@@ -26,7 +26,8 @@ def test_library_exports_every_declared_symbol():
 def test_header_enums_match_python_constants():
     header = (ROOT / "include" / "mxgemm.h").read_text()
     for name in ["MX_E4M3", "MX_E5M2", "MX_E2M1", "MX_E8M0", "MX_F32", "MX_BF16", "MX_F16", "MX_I32",
-                 "MX_SCALE_2D", "MX_SCALE_SWIZZLE_32_4_4", "MX_SCALE_NATIVE", "MX_KERNEL_AUTO", "MX_KERNEL_GENERIC",
+                 "MX_SCALE_2D", "MX_SCALE_SWIZZLE_32_4_4", "MX_SCALE_NATIVE", "MX_SCALE_NATIVE32", "MX_OPERAND_A",
+                 "MX_OPERAND_B", "MX_KERNEL_AUTO", "MX_KERNEL_GENERIC",
                  "MX_KERNEL_MFMA_128x128", "MX_KERNEL_MFMA_256x256", "MX_KERNEL_MFMA_256x256_W4", "MX_KERNEL_DECODE", "MX_KERNEL_MFMA_PINGPONG", "MX_KERNEL_MFMA_PINGPONG32", "MX_KERNEL_MFMA_W4_PERSISTENT",
                  "MX_ERR_INVALID", "MX_ERR_SHAPE", "MX_ERR_DTYPE", "MX_ERR_LAYOUT", "MX_ERR_WORKSPACE",
                  "MX_ERR_DEVICE", "MX_ERR_LAUNCH"]:

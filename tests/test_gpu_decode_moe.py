@@ -140,7 +140,7 @@ def test_grouped_gemm_routed_weight_replicas1_and_padded_ids(ct, dev, kernel):
     # pre-packed expert scales give the same bits
     if kernel != "generic":
         C2 = torch.zeros_like(C)
-        ct.invoke_fused_moe_scaled(a.storage, a.scale_t, W, ct.pack_scales(Ws), C2, wts.to(dev), sid, eid, True, 1,
+        ct.invoke_fused_moe_scaled(a.storage, a.scale_t, W, ct.pack_scales(Ws, operand="b", kernel=kernel), C2, wts.to(dev), sid, eid, True, 1,
                                    256, kernel=kernel)
         assert torch.equal(C, C2)
         # bf16 output (the full-vector store path of the scatter epilogue where the tile's columns are inside N)

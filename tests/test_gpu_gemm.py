@@ -93,7 +93,8 @@ def test_prepacked_scales_and_accumulate(ct, dev, kernel):
     a = randn_operand(256, 512, O.E4M3, 41, dev)
     b = randn_operand(384, 512, O.E4M3, 42, dev)
     ref = oracle_matmul(a, b)
-    pa, pb = ct.pack_scales(a.scale_t), ct.pack_scales(b.scale_t.T, transposed=True)
+    pa = ct.pack_scales(a.scale_t, operand="a", kernel=kernel)
+    pb = ct.pack_scales(b.scale_t.T, transposed=True, operand="b", kernel=kernel)
     c = ct.block_scaled_matmul(a.storage, pa, b.storage.T, pb, kernel=kernel)
     c_plain = _run(ct, a, b, kernel=kernel)
     assert torch.equal(c, c_plain)

@@ -81,38 +81,71 @@ def test_quantize_dequantize_roundtrip_large(ct, dev):
     assert torch.equal(xq2.view(torch.uint8), q)
 
 
-def _native_layout_loops(scales: np.ndarray) -> np.ndarray:
-    """Plain-numpy statement of the native scale layout: dword [I/4][Q][lane][I%4], byte t = scale of row
-    16 I + lane%16, block (4Q + t)*4 + lane/16; padding byte 127."""
+def _bperm_row(j: int, c: int) -> int:
+    """Row of a 64-row group that the 16x16x128 kernels feed to the instruction as operand row c of tile j."""
+    return 32 * (j // 2) + 8 * (c // 4) + 4 * (j % 2) + c % 4
+
+
+def _native_layout_loops(scales: np.ndarray, target: str = "a") -> np.ndarray:
+    """Plain-numpy statement of the native scale layouts, element by element.  16 bytes per (64-row group G,
+    K-quad Q, lane = c + 16 g), holding the scales of K block (4 Q + t) * 4 + g for t = 0..3 and four rows:
+      "a":      byte [t][b] = row 64 G + 16 b + c        (MX_SCALE_NATIVE, A operand)
+      "b":      byte [t][b] = row 64 G + bperm_row(b, c) (MX_SCALE_NATIVE, B operand)
+      "tile32": byte [b][t] = row 64 G + 16 b + c        (MX_SCALE_NATIVE32)
+    padding byte 127."""
     R, KB = scales.shape
     R64, KQ = -(-R // 64), -(-KB // 16)
     out = np.full((R64, KQ, 64, 4, 4), 127, dtype=np.uint8)
-    for row in range(R):
-        for kb in range(KB):
-            I, r = divmod(row, 16)
-            ks, g = divmod(kb, 4)
-            Q, t = divmod(ks, 4)
-            out[I // 4, Q, g * 16 + r, I % 4, t] = scales[row, kb]
+    for G in range(R64):
+        for b in range(4):
+            for c in range(16):
+                row = 64 * G + (_bperm_row(b, c) if target == "b" else 16 * b + c)
+                if row >= R:
+                    continue
+                for kb in range(KB):
+                    ks, g = divmod(kb, 4)
+                    Q, t = divmod(ks, 4)
+                    if target == "tile32":
+                        out[G, Q, g * 16 + c, b, t] = scales[row, kb]
+                    else:
+                        out[G, Q, g * 16 + c, t, b] = scales[row, kb]
     return out.reshape(-1)
 
 
+_PACK_KW = {"a": dict(operand="a"), "b": dict(operand="b"), "tile32": dict(operand="a", kernel="pingpong32")}
+
+
+@pytest.mark.parametrize("target", ["a", "b", "tile32"])
 @pytest.mark.parametrize("R,K", [(64, 512), (100, 160), (256, 1024), (16, 32), (128, 128), (384, 2048)])
-def test_pack_scales_layout_all_sources_agree(ct, dev, R, K):
-    """Element-by-element statement of the layout, and the same bytes from every source form: row-major,
+def test_pack_scales_layout_all_sources_agree(ct, dev, R, K, target):
+    """Element-by-element statement of each layout, and the same bytes from every source form: row-major,
     transposed (how B_scale is passed) and the 4-D swizzle_32_4_4 tensor."""
     rng = np.random.default_rng(R + K)
     s = rng.integers(0, 255, (R, K // 32), dtype=np.uint8)
     t = torch.from_numpy(s).to(dev)
-    p = ct.pack_scales(t.view(torch.float8_e8m0fnu))
-    want = _native_layout_loops(s)
+    kw = _PACK_KW[target]
+    p = ct.pack_scales(t.view(torch.float8_e8m0fnu), **kw)
+    want = _native_layout_loops(s, target)
     got = p.data.cpu().numpy()[:want.size]
     assert np.array_equal(got, want)
     # transposed source (how B_scale is passed) gives the same bytes
-    p2 = ct.pack_scales(t.T.contiguous().view(torch.float8_e8m0fnu), transposed=True)
+    p2 = ct.pack_scales(t.T.contiguous().view(torch.float8_e8m0fnu), transposed=True, **kw)
     assert torch.equal(p.data, p2.data)
     if R % 128 == 0 and (K // 32) % 4 == 0:
-        p3 = ct.pack_scales(ct.swizzle_32_4_4(t))
+        p3 = ct.pack_scales(ct.swizzle_32_4_4(t), **kw)
         assert torch.equal(p.data, p3.data)
+
+
+def test_pack_scales_operand_defaults_and_mismatch(ct, dev):
+    s = torch.randint(100, 140, (128, 16), dtype=torch.uint8, device=dev)
+    assert ct.pack_scales(s).operand == "a" and ct.pack_scales(s.T.contiguous(), transposed=True).operand == "b"
+    assert ct.pack_scales(s.reshape(2, 64, 16)).operand == "b"          # a batch of expert weights
+    a = torch.zeros((128, 512), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    with pytest.raises(ValueError, match="packed for operand"):
+        ct.block_scaled_matmul(a, ct.pack_scales(s, operand="b"), a.T, ct.pack_scales(s, operand="b"))
+    with pytest.raises(ct.TileTypeError, match="native-layout scales of kind"):
+        ct.block_scaled_matmul(a, ct.pack_scales(s, operand="a", kernel="pingpong32"), a.T,
+                               ct.pack_scales(s, operand="b", kernel="pingpong32"), kernel="mfma128")
 
 
 def test_swizzle_roundtrip_device(ct, dev):
@@ -123,46 +156,53 @@ def test_swizzle_roundtrip_device(ct, dev):
     assert torch.equal(ct.unswizzle_32_4_4(sw), s)
 
 
-def _native_layout(sc: np.ndarray) -> np.ndarray:
-    """The packed layout, restated: dword [I / 4][Q][lane][I % 4] holds, in byte t, the scale of row
-    16 I + lane % 16 for K block (4 Q + t) * 4 + lane / 16; rows padded to 64 and blocks to 16 with 127."""
+def _native_layout(sc: np.ndarray, target: str = "a") -> np.ndarray:
+    """The packed layouts restated with array slicing (see _native_layout_loops for the element-wise form); rows
+    padded to 64 and K blocks to 16 with 127."""
     rows, KB = sc.shape
     R, KQ = -(-rows // 64) * 64, -(-KB // 16)
     full = np.full((R, KQ * 16), 127, dtype=np.uint8)
     full[:rows, :KB] = sc
-    out = np.zeros((R // 64, KQ, 64, 4, 4), dtype=np.uint8)   # [I/4][Q][lane][I%4][t]
+    out = np.zeros((R // 64, KQ, 64, 4, 4), dtype=np.uint8)   # [G][Q][lane][first index][second index]
     for lane in range(64):
-        r, g = lane % 16, lane // 16
-        for i4 in range(4):
+        c, g = lane % 16, lane // 16
+        for b in range(4):
+            row = _bperm_row(b, c) if target == "b" else 16 * b + c
             for t in range(4):
-                out[:, :, lane, i4, t] = full[i4 * 16 + r::64, :].reshape(R // 64, KQ, 16)[:, :, 4 * t + g]
+                v = full[row::64, :].reshape(R // 64, KQ, 16)[:, :, 4 * t + g]
+                if target == "tile32":
+                    out[:, :, lane, b, t] = v
+                else:
+                    out[:, :, lane, t, b] = v
     return out.reshape(-1)
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("rows,KB", [(64, 16), (100, 37), (256, 256), (1, 1), (130, 5)])
 @pytest.mark.parametrize("form", ["row_major", "transposed", "sliced", "batched"])
-def test_pack_scales_layout(ct, dev, rows, KB, form):
+@pytest.mark.parametrize("target", ["a", "b", "tile32"])
+def test_pack_scales_layout(ct, dev, rows, KB, form, target):
     """mx_pack_scales against a restatement of the layout, for every source form the staging code
     distinguishes (16-byte loads along K or along rows, misaligned sources, batches)."""
     rng = np.random.default_rng(rows * 1000 + KB)
+    kw = _PACK_KW[target]
     if form == "batched":
         sc = rng.integers(0, 255, size=(3, rows, KB), dtype=np.uint8)
-        got = ct.pack_scales(torch.from_numpy(sc).to(dev)).data.cpu().numpy()
-        want = np.concatenate([_native_layout(sc[b]) for b in range(3)])
+        got = ct.pack_scales(torch.from_numpy(sc).to(dev), **kw).data.cpu().numpy()
+        want = np.concatenate([_native_layout(sc[b], target) for b in range(3)])
     else:
         sc = rng.integers(0, 255, size=(rows, KB), dtype=np.uint8)
         if form == "row_major":
             t = torch.from_numpy(sc).to(dev)
-            got = ct.pack_scales(t).data.cpu().numpy()
+            got = ct.pack_scales(t, **kw).data.cpu().numpy()
         elif form == "transposed":
             t = torch.from_numpy(np.ascontiguousarray(sc.T)).to(dev)   # [K/32, rows], as B_scale arrives
-            got = ct.pack_scales(t, transposed=True).data.cpu().numpy()
+            got = ct.pack_scales(t, transposed=True, **kw).data.cpu().numpy()
         else:
             big = torch.zeros((rows + 3, KB + 7), dtype=torch.uint8, device=dev)
             big[1:rows + 1, 3:KB + 3] = torch.from_numpy(sc).to(dev)
-            got = ct.pack_scales(big[1:rows + 1, 3:KB + 3]).data.cpu().numpy()
-        want = _native_layout(sc)
+            got = ct.pack_scales(big[1:rows + 1, 3:KB + 3], **kw).data.cpu().numpy()
+        want = _native_layout(sc, target)
     assert np.array_equal(got, want)
 
 
