@@ -141,10 +141,31 @@ def profile_traffic(tag):
         return None
 
 
+def profile_clock(tag):
+    """Shader clock (GHz) the kernel of configuration `tag` sustained in the rocprofv3 counter run kept under
+    profiles/ (line `clock_ghz[tag] = X`: kernel cycles from SQ_BUSY_CYCLES over the kernel's duration); None if
+    no figure is kept there."""
+    try:
+        m = re.search(rf"clock_ghz\[{tag}\]\s*=\s*([0-9.]+)", PROFILE_TRAFFIC.read_text())
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+NOMINAL_CLOCK_GHZ = 2.4   # the clock the dense MFMA peaks are quoted at
+
+
 def roofline(bound, achieved, peak, unit, tag, kernel, w, work):
-    return {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
-            "traffic": profile_traffic(tag), "kernel": kernel, "kernel_ms": w.mean * 1e-3,
-            ("flops_per_launch" if bound == "mfma" else "bytes_per_launch"): work, **w.stats()}
+    r = {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
+         "traffic": profile_traffic(tag), "kernel": kernel, "kernel_ms": w.mean * 1e-3,
+         ("flops_per_launch" if bound == "mfma" else "bytes_per_launch"): work, **w.stats()}
+    if bound == "mfma":
+        # the chip lowers its clock under this load: the fraction of the peak at the clock the kernel actually ran at
+        # (from the counter run under profiles/, like `traffic`) is the share of cycles the matrix pipe was fed
+        clk = profile_clock(tag)
+        r["clock_ghz"] = clk
+        r["frac_at_clock"] = achieved / (peak * clk / NOMINAL_CLOCK_GHZ) if clk else None
+    return r
 
 
 def _quantized(ct, rows, K, fmt, seed, dev, dist, std=1.0, cpu_seeded=True):
@@ -292,35 +313,90 @@ def bench_recorded_4096(ct, O, dev, steps, warmup, check, nsets=4):
         ct.block_scaled_matmul(a_q, a_sw, b_q.T, b_sw, C=c, cache_scales=True)
 
     t_call_cached = _time_events(step_cached, steps, max(warmup, 2 * nsets))
+
+    # the reference's own signature, cutile_block_scaled_matmul(A, A_scale, B, B_scale) -> C (it allocates the fp32
+    # result like the sample does, and keeps the scale re-layout between calls)
+    def step_drop_in(i):
+        a_q, _, b_q, _, a_sw, b_sw, _ = sets[i % nsets]
+        ct.cutile_block_scaled_matmul(a_q, a_sw, b_q.T, b_sw)
+
+    t_call_drop_in = _time_events(step_drop_in, steps, max(warmup, 2 * nsets))
     packed = [(s[0], ct.pack_scales(s[1], operand="a"), s[2].T, ct.pack_scales(s[3], operand="b"), s[6]) for s in sets]
     w = measure(lambda k: [t * 1e3 for t in ct.bench_block_scaled_matmul(packed, warmup=3, iters=k)], batch=10)
     flops = 2.0 * M * N * K
     return {"call_us_incl_scale_relayout": t_call * 1e6, "tflops": flops / t_call * 1e-12,
-            "call_us_cached_scales": t_call_cached * 1e6,
+            "call_us_cached_scales": t_call_cached * 1e6, "call_us_drop_in_signature": t_call_drop_in * 1e6,
             "gemm_kernel_us": w.mean, "gemm_kernel_tflops": flops / w.mean * 1e-6, **w.stats(),
             "reference_recorded_us_b200": 71.379, "reference_recorded_ci_us_b200": 0.294,
             "rel_fro_vs_oracle": err}
 
 
-def bench_decode(ct, O, dev, steps, warmup, check, nsets=8):
-    """Decode-shaped mixed GEMM: X MXFP8 (32, 8192) x W MXFP4 (28672, 8192)^T, bf16 out.  HBM bound; the
-    121 MiB working set fits in the Infinity Cache, so 8 weight sets are rotated."""
-    M, N, K = 32, 28672, 8192
+def bench_shape(ct, O, dev, M, N, K, check, kernels=("auto", "mfma128", "pingpong"), swizzled=True, nsets=3):
+    """One problem of the reference's own benchmark list (test/bench_matmul.py:419-425 shapes, :98-112 check): MXFP8
+    E4M3, scales in the swizzle_32_4_4 form, fp32 output, checked against the oracle before timing.  Reports a call
+    through the drop-in signature (scale re-layout inside) and the GEMM kernel alone for the kernel MX_KERNEL_AUTO
+    picks and for each candidate kernel, so that the cost of the selection rule is on record."""
+    nsets = max(nsets, min(8, -(-(300 << 20) // (M * K + N * K + M * N * 4))))   # rotate more than the Infinity Cache
+    sets = []
+    for i in range(nsets):
+        a_q, a_s = _quantized(ct, M, K, torch.float8_e4m3fn, 5001 + 2 * i, dev, "randn", cpu_seeded=(i == 0))
+        b_q, b_s = _quantized(ct, N, K, torch.float8_e4m3fn, 5002 + 2 * i, dev, "randn", cpu_seeded=(i == 0))
+        sw = swizzled and M % 128 == 0 and N % 128 == 0 and (K // 32) % 4 == 0
+        sets.append((a_q, a_s, b_q, b_s, ct.swizzle_32_4_4(a_s) if sw else a_s, ct.swizzle_32_4_4(b_s) if sw else b_s.T,
+                     torch.empty((M, N), dtype=torch.float32, device=dev)))
+    err = None
+    if check:
+        a_q, a_s, b_q, b_s, a_sw, b_sw, c = sets[0]
+        ct.block_scaled_matmul(a_q, a_sw, b_q.T, b_sw, C=c)
+        rows = torch.arange(0, M, max(1, M // 32))[:32]
+        err = _check_rows(O, c, _oracle_rows(O, a_q, a_s, b_q, b_s, rows, O.E4M3, O.E4M3), rows, 1e-3, f"{M}x{N}x{K}")
+
+    def step(i):
+        a_q, _, b_q, _, a_sw, b_sw, c = sets[i % nsets]
+        ct.block_scaled_matmul(a_q, a_sw, b_q.T, b_sw, C=c)
+
+    t_call = _time_events(step, 50, 10)
+    flops = 2.0 * M * N * K
+    out = {"M": M, "N": N, "K": K, "call_us_incl_scale_relayout": t_call * 1e6, "rel_fro_vs_oracle": err, "kernel_us": {}}
+    packed = [(s[0], ct.pack_scales(s[1], operand="a"), s[2].T, ct.pack_scales(s[3], operand="b"), s[6]) for s in sets]
+    for kern in kernels:
+        try:
+            w = measure(lambda k: [t * 1e3 for t in ct.bench_block_scaled_matmul(packed, warmup=3, iters=k, kernel=kern)], batch=10)
+        except (ValueError, TypeError, RuntimeError) as e:      # a kernel that does not take this shape
+            out["kernel_us"][kern] = {"error": str(e)[:120]}
+            continue
+        out["kernel_us"][kern] = {**w.stats(), "tflops": flops / w.mean * 1e-6}
+        if kern == "auto":
+            out["roofline"] = roofline("mfma", flops / w.mean * 1e-6, PEAK_TFLOPS["mxfp8"], "TFLOP/s", "none",
+                                       "kernel chosen by MX_KERNEL_AUTO", w, flops)
+    best = min((v["mean_us"] for v in out["kernel_us"].values() if "mean_us" in v), default=None)
+    auto = out["kernel_us"].get("auto", {}).get("mean_us")
+    out["auto_over_best"] = auto / best if auto and best else None
+    return out
+
+
+def bench_decode(ct, O, dev, steps, warmup, check, M=32, N=28672, K=8192, nsets=8):
+    """Decode-shaped mixed GEMM: X MXFP8 (M, K) x W MXFP4 (N, K)^T, bf16 out; the headline shape is 32 x 28672 x 8192.
+    HBM bound; its 121 MiB working set fits in the Infinity Cache, so several weight sets are rotated.  Shapes the
+    skinny-M kernel does not take (M > 32) run on what MX_KERNEL_AUTO picks, with the weight scales packed once."""
     x_q, x_s = _quantized(ct, M, K, torch.float8_e4m3fn, 2001, dev, "randn")
+    nsets = max(nsets, -(-(300 << 20) // (N * K // 2)))
     ws = []
     for i in range(nsets):
         w_q, w_s = _quantized(ct, N, K, "e2m1", 2002 + i, dev, "randn", std=0.02, cpu_seeded=(i == 0))
-        ws.append((w_q, w_s, torch.empty((M, N), dtype=torch.bfloat16, device=dev)))
+        ws.append((w_q, w_s, torch.empty((M, N), dtype=torch.bfloat16, device=dev),
+                   w_s.T if M <= 32 else ct.pack_scales(w_s, operand="b")))
     err = None
     if check:
-        w_q, w_s, c = ws[0]
-        ct.block_scaled_matmul(x_q, x_s, w_q.T, w_s.T, b_format="e2m1", C=c)
-        ref = _oracle_rows(O, x_q, x_s, w_q, w_s, torch.arange(M), O.E4M3, O.E2M1)
-        err = _check_rows(O, c, ref, torch.arange(M), 8e-3, "decode 32x28672x8192")
+        w_q, w_s, c, w_sc = ws[0]
+        ct.block_scaled_matmul(x_q, x_s, w_q.T, w_sc, b_format="e2m1", C=c)
+        rows = torch.arange(min(M, 32))
+        ref = _oracle_rows(O, x_q, x_s, w_q, w_s, rows, O.E4M3, O.E2M1)
+        err = _check_rows(O, c, ref, rows, 8e-3, f"decode {M}x{N}x{K}")
 
     def step(i):
-        w_q, w_s, c = ws[i % nsets]
-        ct.block_scaled_matmul(x_q, x_s, w_q.T, w_s.T, b_format="e2m1", C=c)
+        w_q, w_s, c, w_sc = ws[i % nsets]
+        ct.block_scaled_matmul(x_q, x_s, w_q.T, w_sc, b_format="e2m1", C=c)
 
     t_wall = _time_wall(step, steps, warmup)
     # The kernel runs ~20 us, less than the host needs to issue a launch from Python, so the kernel's own
@@ -335,7 +411,7 @@ def bench_decode(ct, O, dev, steps, warmup, check, nsets=8):
     # one sample = one replay (per_graph launches back to back on the stream) between a pair of events, / per_graph
     rb = _events_batch(lambda i: graph.replay())
     w = measure(lambda k: [t / per_graph for t in rb(k)])
-    nbytes = M * K + M * K // 32 + N * K // 2 + N * K // 32 + M * N * 2     # 126 885 888
+    nbytes = M * K + M * K // 32 + N * K // 2 + N * K // 32 + M * N * 2     # 126 885 888 for the headline shape
     return {"ms_per_step": t_wall * 1e3, "kernel": w, "gbs": nbytes / (w.mean * 1e-6) * 1e-9,
             "gbs_wall": nbytes / t_wall * 1e-9, "bytes": nbytes, "rel_fro_vs_oracle": err}
 
@@ -453,7 +529,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c5,r4096 (default: all)")
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c5,r4096,shapes (default: all)")
     ap.add_argument("--kernel", default="auto",
                     help="kernel of the square GEMM legs: auto, pingpong, pingpong32, w4p, mfma256, mfma256w4, mfma128 "
                          "(the counter comparisons under profiles/ are runs of this file with this option)")
@@ -488,7 +564,7 @@ def main():
         dst.copy_(src)          # 256 MiB read + 256 MiB written by one elementwise copy kernel
         _sync()
         del src, dst
-    want = set(filter(None, a.only.split(","))) or {"c2", "c3", "c4", "c5", "r4096"}
+    want = set(filter(None, a.only.split(","))) or {"c2", "c3", "c4", "c5", "r4096", "shapes"}
     check = not a.no_check
     kname = {"auto": "gemm_pp_kernel", "pingpong": "gemm_pp_kernel", "pingpong32": "gemm_pp32_kernel",
              "w4p": "gemm_w4_kernel", "mfma256": "gemm_kernel<256x256,8 waves>", "mfma256w4": "gemm_kernel<256x256,4 waves>",
@@ -506,6 +582,15 @@ def main():
     if "r4096" in want:
         extra["recorded_problem_mxfp8_4096_swizzled_fp32"] = bench_recorded_4096(ct, O, dev, a.steps, a.warmup, check)
         torch.cuda.empty_cache()
+    if "shapes" in want:
+        # the reference benchmark's other two problems (test/bench_matmul.py:419-425) and two mid-size points: one
+        # with few tiles and a long K, one with 400 tiles of 256 x 256 (1.56 rounds of the 256 CUs)
+        for name, (M, N, K) in (("ref_bench_1024", (1024, 1024, 1024)),
+                                ("ref_bench_12288x4096x2560", (12288, 4096, 2560)),
+                                ("mid_2048x2048x8192", (2048, 2048, 8192)),
+                                ("mid_5120", (5120, 5120, 5120))):
+            extra[name] = bench_shape(ct, O, dev, M, N, K, check)
+            torch.cuda.empty_cache()
     if "c3" in want:
         r = bench_decode(ct, O, dev, max(a.steps, 50), a.warmup, check)
         extra["c3_decode_m32"] = {"gbs_wall_clock": r["gbs_wall"], "ms_per_step": r["ms_per_step"],
@@ -513,6 +598,16 @@ def main():
                                   "roofline": roofline("hbm", r["gbs"], PEAK_HBM_GBS, "GB/s", "c3",
                                                        "decode_kernel<e4m3,16,bf16>", r["kernel"], r["bytes"])}
         torch.cuda.empty_cache()
+        # beyond the headline shape: K longer than one launch of the skinny-M kernel takes (the down-projection
+        # of the MoE layer of the grouped workload), and 32 < M <= 128 on the same weights (tiled kernels)
+        for name, (M, N, K) in (("decode_m32_k14336", (32, 4096, 14336)), ("decode_m64", (64, 28672, 8192)),
+                                ("decode_m128", (128, 28672, 8192))):
+            r = bench_decode(ct, O, dev, 50, a.warmup, check, M=M, N=N, K=K)
+            extra[name] = {"M": M, "N": N, "K": K, "rel_fro_vs_oracle": r["rel_fro_vs_oracle"],
+                           "call_us": r["kernel"].mean, "gbs": r["gbs"], "frac_of_hbm_peak": r["gbs"] / PEAK_HBM_GBS,
+                           "bytes_per_launch": r["bytes"], **r["kernel"].stats()}
+            del r
+            torch.cuda.empty_cache()
     if "c5" in want:
         r = bench_moe(ct, O, dev, a.steps, a.warmup, check, full_forward=not a.no_moe_forward)
         e5 = {"tflops": r["tflops"], "ms_per_step": r["ms_per_step"], "padded_rows": r["padded_rows"],

@@ -48,6 +48,18 @@ inline int native_layout_of(int kernel) {
 }
 inline bool is_native(int layout) { return layout == MX_SCALE_NATIVE || layout == MX_SCALE_NATIVE32; }
 
+// The decode kernel takes K up to kDecodeChunk per launch; a longer K runs as one launch per chunk, the chunks adding
+// up in an fp32 buffer of the workspace that a last pass converts into C.
+constexpr int64_t kDecodeChunk = 8192;
+inline bool decode_shape(int64_t M, int64_t N, int64_t K) { return M >= 1 && M <= 32 && K % 512 == 0 && N % 16 == 0; }
+// workspace of that buffer; depends on (M, N, K, opts) only, so it is also counted for problems whose operand types
+// then send them to another kernel
+inline int64_t decode_partial_bytes(int64_t M, int64_t N, int64_t K, const mx_gemm_opts& o) {
+  if ((o.kernel != MX_KERNEL_AUTO && o.kernel != MX_KERNEL_DECODE) || !decode_shape(M, N, K) || K <= kDecodeChunk)
+    return 0;
+  return round256(M * N * 4);
+}
+
 const mx_gemm_opts kDefaultOpts = {sizeof(mx_gemm_opts), 0, MX_SCALE_2D, MX_SCALE_2D, MX_KERNEL_AUTO, 32, 0, 0};
 
 // Number of K-slices for a problem that ends up on a one-tile MFMA kernel (1 = no split).  Depends only on
@@ -153,7 +165,8 @@ int64_t mx_packed_scale_bytes(int64_t rows, int64_t K) {
 int64_t mx_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, const mx_gemm_opts* opts) {
   const mx_gemm_opts& o = opts ? *opts : kDefaultOpts;
   if (o.kernel == MX_KERNEL_GENERIC) return 0;
-  int64_t b = 0;
+  if (o.kernel == MX_KERNEL_DECODE) return decode_partial_bytes(M, N, K, o);
+  int64_t b = decode_partial_bytes(M, N, K, o);
   const int S = plan_k_splits(M, N, K, o);
   if (S > 1) {   // per-slice packed scales and the fp32 partial products
     b += S * (mx_packed_scale_bytes(M, K / S) + mx_packed_scale_bytes(N, K / S));
@@ -361,7 +374,7 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
     if (why) kernel = MX_KERNEL_GENERIC;
     else if (M <= 32 && A->dtype != MX_E2M1 && B->dtype == MX_E2M1 && o.a_scale_layout == MX_SCALE_2D &&
              o.b_scale_layout == MX_SCALE_2D && Bs->stride[0] == 1 && As->stride[1] == 1 && K % 512 == 0 &&
-             K <= 8192 && N % 16 == 0 && Bs->stride[1] % 16 == 0 && ((uintptr_t)Bs->ptr) % 16 == 0 &&
+             N % 16 == 0 && Bs->stride[1] % 16 == 0 && ((uintptr_t)Bs->ptr) % 16 == 0 &&
              N * b_ld < ((int64_t)1 << 31) && As->stride[0] % 16 == 0 && ((uintptr_t)As->ptr) % 16 == 0)
       kernel = MX_KERNEL_DECODE;
     else if (big_tile_problem(M, N)) kernel = big_tile_kernel();
@@ -423,15 +436,32 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
       return set_error(MX_ERR_LAYOUT, "the decode kernel reads K-contiguous 2-D scales in place");
     if (A->dtype == MX_E2M1 || B->dtype != MX_E2M1)
       return set_error(MX_ERR_DTYPE, "the decode kernel takes 8-bit activations and FP4 weights");
-    if (K % 512 != 0 || K > 8192 || N % 16 != 0)
-      return set_error(MX_ERR_SHAPE, "the decode kernel needs K %% 512 == 0, K <= 8192 and N %% 16 == 0");
+    if (K % 512 != 0 || N % 16 != 0)
+      return set_error(MX_ERR_SHAPE, "the decode kernel needs K %% 512 == 0 and N %% 16 == 0");
     DecodeArgs d = {};
     d.X = (const uint8_t*)A->ptr; d.Xs = (const uint8_t*)As->ptr;
     d.W = (const uint8_t*)B->ptr; d.Ws = (const uint8_t*)Bs->ptr; d.C = C->ptr;
     d.M = (int32_t)M; d.N = (int32_t)N; d.K = (int32_t)K;
     d.ldx = a_ld; d.ldxs = As->stride[0]; d.ldw = b_ld; d.ldws = Bs->stride[1]; d.ldc = C->stride[0];
     d.x_fmt = A->dtype; d.w_fmt = B->dtype; d.c_dtype = C->dtype; d.accumulate = o.accumulate;
-    return launch_gemm_decode(d, (hipStream_t)stream);
+    if (K <= kDecodeChunk) return launch_gemm_decode(d, (hipStream_t)stream);
+    // a longer K (the down-projection of an MoE layer, K = 14336 / 28672): chunks of kDecodeChunk elements, each
+    // streaming its part of the weights once, summed in fp32 in the workspace in chunk order
+    const int64_t need = decode_partial_bytes(M, N, K, o);
+    if (!workspace || workspace_bytes < need)
+      return set_error(MX_ERR_WORKSPACE, "workspace of %lld bytes required, %lld given", (long long)need,
+                       (long long)workspace_bytes);
+    if (((uintptr_t)workspace) % 256 != 0) return set_error(MX_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+    for (int64_t k0 = 0; k0 < K; k0 += kDecodeChunk) {
+      DecodeArgs c = d;
+      c.X = d.X + k0; c.Xs = d.Xs + k0 / 32;          // 8-bit activations: one byte per element
+      c.W = d.W + k0 / 2; c.Ws = d.Ws + k0 / 32;      // FP4 weights: two elements per byte
+      c.K = (int32_t)(K - k0 < kDecodeChunk ? K - k0 : kDecodeChunk);
+      c.C = workspace; c.ldc = N; c.c_dtype = MX_F32; c.accumulate = k0 > 0;
+      if (int rc = launch_gemm_decode(c, (hipStream_t)stream)) return rc;
+    }
+    return launch_splitk_reduce((const float*)workspace, 1, M, N, C->ptr, C->stride[0], C->dtype, o.accumulate,
+                                (hipStream_t)stream);
   }
 
   // ---- MFMA path: bring the scales into the native layout if they are not ----------------------------

@@ -121,7 +121,9 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
   const bool with_scales = wave < Cf::S_INSTR;
 
   // ---- per-lane DMA offsets inside a tile --------------------------------------------------------------
-  const uint32_t wbytes = (uint32_t)((int64_t)d.N * d.ldw), sbytes = (uint32_t)((int64_t)d.N * d.ldws);
+  // (descriptor ranges end with the last row's last byte of this K range: the operands may be K-chunks of wider rows)
+  const uint32_t wbytes = (uint32_t)((int64_t)(d.N - 1) * d.ldw + d.K / 2);
+  const uint32_t sbytes = (uint32_t)((int64_t)(d.N - 1) * d.ldws + d.K / 32);
   const int rl = lane / Cf::LPR;                 // row of the lane inside one DMA instruction
   const uint32_t row_off = (uint32_t)(rl * d.ldw);
   const uint32_t chunk_off = (uint32_t)((((lane % Cf::LPR) ^ rl) << 4) + q * Cf::SLB);   // SLB: no bits below 512
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
     issue(0, 1);                                       // tile i lives in slot (i + 1) % 2
     lds_u8* const xst = smem + Cf::XSTAGE_OFF + wave * (Cf::XNB * 4096);
     lds_u8* const xsst = smem + Cf::XSCALE_OFF + wave * 1024;
-    const uint32_t xbytes = (uint32_t)((int64_t)d.M * d.ldx);
+    const uint32_t xbytes = (uint32_t)((int64_t)(d.M - 1) * d.ldx + d.K);
     uint32_t xvo[4];                                  // lane offsets of the 4 DMA instructions of a round
     int xcb[4];
 #pragma unroll
@@ -185,7 +187,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(const DecodeArgs d)
       constexpr int LPRS = SPW * 4 / 16;              // lanes per row
       const int srw = lane / LPRS;
       const bool sok = srw < 16 && 16 * mh + srw < d.M && q * SPW * 4 + (lane % LPRS) * 16 < d.K / 32;
-      issue_xs_dma(d.Xs, (uint32_t)((int64_t)d.M * d.ldxs), xsst,
+      issue_xs_dma(d.Xs, (uint32_t)((int64_t)(d.M - 1) * d.ldxs + d.K / 32), xsst,
                    sok ? (uint32_t)(srw * d.ldxs + (lane % LPRS) * 16) : kOob, 16 * mh * (int)d.ldxs + q * SPW * 4);
     }
 #pragma unroll

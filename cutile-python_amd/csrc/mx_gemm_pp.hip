@@ -187,13 +187,13 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_void*)(base + q * 4096), 16, v, ka, 0, 0);
     }
   };
-  auto issue_b = [&](int sl, int bbuf) {
+  auto issue_b = [&](int sl, int bbuf, int q0 = 0, int q1 = P::BL) {   // DMA instructions q0 .. q1 - 1
     if constexpr (TEAM == 1) {
       lds_u8* const base = smem + P::B_BASE + bbuf * C::B_STAGE + wn0 * C::B_RB;
       const int kb = sl * C::B_RB;
       const int klim = sl < nstages ? Kb_b - kb : 0;
 #pragma unroll
-      for (int q = 0; q < BL; ++q) {
+      for (int q = q0; q < q1; ++q) {
         const int col = b_col(q);
         const uint32_t v = (KTAIL && col >= klim) ? kOobOffset : b_voff[q];
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_void*)(base + q * 1024), 16, v, kb, 0, 0);
@@ -349,19 +349,33 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     issue_a(sl_eff, abuf2);
     v8i bf[C::KSUB][4], af[C::KSUB][8];
     if (!(GROUPED && skip_cur)) {
+      // B tiles 0, 1 (rows 0 .. 31 of the wave's 64), then tiles 2, 3, then the early A tiles: LDS returns reads in
+      // order, so the DMA that refills the first half of the B rows can go as soon as the first group is back
 #pragma unroll
-      for (int kk = 0; kk < C::KSUB; ++kk) {
+      for (int h = 0; h < 2; ++h) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) bf[kk][j] = load_frag<C::B_RB, C::B_EB>(btile, bperm_tile_off(j), kk, gq, swb);
+        for (int kk = 0; kk < C::KSUB; ++kk)
+#pragma unroll
+          for (int j = 2 * h; j < 2 * h + 2; ++j) bf[kk][j] = load_frag<C::B_RB, C::B_EB>(btile, bperm_tile_off(j), kk, gq, swb);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int kk = 0; kk < C::KSUB; ++kk)
 #pragma unroll
         for (int i = 0; i < EARLY; ++i) af[kk][i] = load_frag<C::A_RB, C::A_EB>(atile, 16 * i, kk, gq, swa);
-      }
+      __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (TEAM == 1) {
       // the B buffer of this stage is free once this wave's own reads have returned
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      constexpr int NBH = 2 * C::KSUB * (C::B_EB == 8 ? 2 : 1);       // LDS reads of two B tiles
+      constexpr int NAE = EARLY * C::KSUB * (C::A_EB == 8 ? 2 : 1);   // LDS reads of the early A tiles
+      asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(NBH + NAE) : "memory");
       __builtin_amdgcn_sched_barrier(0);
-      issue_b(sl_eff, bbuf);
+      issue_b(sl_eff, bbuf, 0, BL / 2);
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(NAE) : "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      issue_b(sl_eff, bbuf, BL / 2, BL);
       // everything older than this phase's loads has landed: A and B of stage s + 1 (the scale loads issued
       // at the start of this phase are younger than those and may stay in flight; the MFMA phase waits for them)
       constexpr int younger = (t0 == 0) ? NSC : 0;
@@ -381,11 +395,11 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
         }
       __builtin_amdgcn_sched_barrier(0);
     };
-    auto mfma_pair = [&](int i0) {
+    auto mfma_pair = [&](int i0, int n = 2) {   // row tiles i0 .. i0 + n - 1
 #pragma unroll
       for (int kk = 0; kk < C::KSUB; ++kk) {
 #pragma unroll
-        for (int i = i0; i < i0 + 2; ++i) {
+        for (int i = i0; i < i0 + n; ++i) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             acc[i][j] = mfma_scaled<C::BF, C::AF>(bf[kk][j], af[kk][i], acc[i][j], j, sb[t0 + kk], i % 4,
@@ -399,6 +413,14 @@ __device__ __forceinline__ void pp_body(const GemmArgs& g, lds_u8* const smem, c
     if (!(GROUPED && skip_cur)) {
 #pragma unroll
       for (int ip = 0; ip < 8; ip += 2) {
+        if (ip == 0) {
+          // the phase opens with MFMAs, not with LDS read issue: the matrix pipe restarts that much sooner after the
+          // hand-over, and the reads issue while the first MFMAs run
+          mfma_pair(0, 1);
+          read_pair(EARLY);
+          mfma_pair(1, 1);
+          continue;
+        }
         if (ip + EARLY < 8) read_pair(ip + EARLY);
         mfma_pair(ip);
       }
@@ -447,8 +469,7 @@ __global__ __launch_bounds__(512) void gemm_pp_kernel(const GemmArgs g) {
   const TileWalk walk = make_tile_walk(g.M, g.N);
   if (walk.first >= walk.end) return;   // cannot happen with the grids the launcher picks
   const int ksteps = (g.K + 127) / 128;
-  // (uniform.  The MXFP4 instance keeps the one masked body: with two bodies in the kernel the register allocator
-  // spills in its stage loop.)
+  // (uniform.  The MXFP4 instance keeps the one masked body: a second, unmasked one measured no faster on it.)
   const bool ktail = C::KSUB != 1 || g.K % 128 != 0 || ksteps < 2;
   if (ktail) {
     if (wave < 4)

@@ -2,13 +2,15 @@
 from __future__ import annotations
 
 import ctypes
+import os
 import pathlib
 import threading
 
 import torch
 
 _HERE = pathlib.Path(__file__).resolve().parent
-LIB_PATH = _HERE / "libmxgemm.so"
+# the library built in-tree; MXGEMM_LIB names another build of it (for example one with other compiler flags)
+LIB_PATH = pathlib.Path(os.environ["MXGEMM_LIB"]) if os.environ.get("MXGEMM_LIB") else _HERE / "libmxgemm.so"
 
 # ---- constants mirrored from include/mxgemm.h -------------------------------------------------
 MX_OK = 0

@@ -459,8 +459,13 @@ def grouped_block_scaled_matmul(As, A_scales, Bs, B_scales, *, out_dtype: torch.
 
 
 def cutile_block_scaled_matmul(A, A_scale, B, B_scale) -> torch.Tensor:
-    """Exact signature of the reference sample wrapper (fp32 result)."""
-    return block_scaled_matmul(A, A_scale, B, B_scale)
+    """Exact signature of the reference sample wrapper (fp32 result, samples/BlockScaledMatMul.py:229-230).  The
+    reference's kernel reads the scales in place; here the MFMA-ready re-layout of each scale tensor is kept with
+    ``cache_scales=True`` (see :func:`block_scaled_matmul`), so repeated calls with the same scale tensors launch the
+    GEMM kernel only.  A cached copy is dropped when torch writes to the tensor (its ``_version`` changes); scale
+    bytes changed behind torch's back (a foreign library writing through the raw pointer) need
+    :func:`clear_scale_cache`, or the general entry :func:`block_scaled_matmul`, which never caches unless asked."""
+    return block_scaled_matmul(A, A_scale, B, B_scale, cache_scales=True)
 
 
 # ==================================================================================================

@@ -13,7 +13,9 @@ pytestmark = pytest.mark.gpu
                                    (17, 4176, 4096), (29, 12320, 8192), (32, 16, 8192), (24, 36864, 4096),
                                    (8, 20480, 4096), (16, 16400, 8192),
                                    # K that ends inside the kernel's K-slices: lanes beyond K fetch nothing
-                                   (32, 1792, 7168), (9, 528, 5120), (32, 272, 3072), (16, 64, 1536), (32, 4112, 6144)])
+                                   (32, 1792, 7168), (9, 528, 5120), (32, 272, 3072), (16, 64, 1536), (32, 4112, 6144),
+                                   # K beyond one launch's 8192: chunks summed in fp32 (down-projection shapes)
+                                   (32, 512, 14336), (5, 1040, 28672), (17, 64, 8704)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=str)
 def test_decode_kernel(ct, dev, M, N, K, out_dtype):
     x = randn_operand(M, K, O.E4M3, 81, dev)
@@ -32,6 +34,22 @@ def test_decode_kernel(ct, dev, M, N, K, out_dtype):
     c3 = ct.block_scaled_matmul(x.storage, x.scale_t, w.storage.T, w.scale_t.T, b_format="e2m1",
                                 out_dtype=out_dtype, kernel="mfma128")
     assert O.rel_fro(c3.float().cpu(), ref) <= (1e-3 if out_dtype == torch.float32 else 8e-3)
+
+
+def test_decode_long_k_accumulate_and_static_scratch(ct, dev):
+    """K = 14336 through the chunked path: C += into bf16 (the conversion pass adds the old C once, in fp32) and the
+    library's static scratch as the chunk buffer."""
+    M, N, K = 24, 336, 14336
+    x = randn_operand(M, K, O.E4M3, 181, dev)
+    w = randn_operand(N, K, O.E2M1, 182, dev, std=0.02)
+    ref = oracle_matmul(x, w)
+    z = torch.randn((M, N), generator=torch.Generator().manual_seed(183)).to(torch.bfloat16)
+    acc = z.to(dev)
+    ct.block_scaled_matmul(x.storage, x.scale_t, w.storage.T, w.scale_t.T, b_format="e2m1", C=acc, accumulate=True)
+    assert O.rel_fro(acc.float().cpu(), ref + z.float()) <= 8e-3
+    c = ct.block_scaled_matmul(x.storage, x.scale_t, w.storage.T, w.scale_t.T, b_format="e2m1", static_scratch=True)
+    c2 = ct.block_scaled_matmul(x.storage, x.scale_t, w.storage.T, w.scale_t.T, b_format="e2m1", kernel="decode")
+    assert torch.equal(c, c2) and O.rel_fro(c.cpu(), ref) <= 1e-3
 
 
 def test_decode_accumulate(ct, dev):

@@ -349,3 +349,23 @@ def test_cached_scale_relayout(ct, dev):
     del a_sw
     ct.clear_scale_cache()
     assert len(ops._SCALE_CACHE._entries) == 0 and n_before >= 2
+
+
+def test_drop_in_signature_caches_scale_relayout(ct, dev):
+    """cutile_block_scaled_matmul(A, A_scale, B, B_scale) -> fp32 C (samples/BlockScaledMatMul.py:229-297): same bits
+    as the general entry, the scale re-layout kept between calls, redone after torch writes to a scale tensor."""
+    from cutile_amd import ops
+    ct.clear_scale_cache()
+    a = randn_operand(512, 768, O.E4M3, 75, dev)
+    b = randn_operand(512, 768, O.E4M3, 76, dev)
+    a_sw, b_sw = ct.swizzle_32_4_4(a.scale_t), ct.swizzle_32_4_4(b.scale_t)     # as the sample passes them
+    want = ct.block_scaled_matmul(a.storage, a_sw, b.storage.T, b_sw)
+    c1 = ct.cutile_block_scaled_matmul(a.storage, a_sw, b.storage.T, b_sw)
+    c2 = ct.cutile_block_scaled_matmul(a.storage, a_sw, b.storage.T, b_sw)
+    assert c1.dtype == torch.float32 and torch.equal(c1, want) and torch.equal(c2, want)
+    assert len(ops._SCALE_CACHE._entries) == 2
+    torch.testing.assert_close(c1.cpu(), oracle_matmul(a, b), atol=1e-4, rtol=1e-3)
+    a_sw.view(torch.uint8).add_(1)                                              # every A scale doubled, through torch
+    c3 = ct.cutile_block_scaled_matmul(a.storage, a_sw, b.storage.T, b_sw)
+    assert torch.equal(c3, want * 2)
+    ct.clear_scale_cache()
