@@ -51,7 +51,14 @@ inline bool is_native(int layout) { return layout == MX_SCALE_NATIVE || layout =
 // The decode kernel takes K up to kDecodeChunk per launch; a longer K runs as one launch per chunk, the chunks adding
 // up in an fp32 buffer of the workspace that a last pass converts into C.
 constexpr int64_t kDecodeChunk = 8192;
-inline bool decode_shape(int64_t M, int64_t N, int64_t K) { return M >= 1 && M <= 32 && K % 512 == 0 && N % 16 == 0; }
+// One launch of it multiplies up to 32 rows of X; more rows run slab by slab, each slab streaming the weights again
+// (the second pass finds most of a weight matrix of up to 256 MiB in the Infinity Cache).  MX_KERNEL_AUTO does that
+// up to kDecodeAutoM rows (measured on 28672 x 8192 FP4 weights: M = 64 takes 2 x 26 us this way against 62 us on the
+// tiled kernel, whose time hardly grows up to M = 128); an explicit MX_KERNEL_DECODE up to kDecodeMaxM.
+constexpr int64_t kDecodeAutoM = 64, kDecodeMaxM = 128;
+inline bool decode_shape(int64_t M, int64_t N, int64_t K) {
+  return M >= 1 && M <= kDecodeMaxM && K % 512 == 0 && N % 16 == 0;
+}
 // workspace of that buffer; depends on (M, N, K, opts) only, so it is also counted for problems whose operand types
 // then send them to another kernel
 inline int64_t decode_partial_bytes(int64_t M, int64_t N, int64_t K, const mx_gemm_opts& o) {
@@ -372,7 +379,7 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
   int kernel = o.kernel;
   if (kernel == MX_KERNEL_AUTO) {
     if (why) kernel = MX_KERNEL_GENERIC;
-    else if (M <= 32 && A->dtype != MX_E2M1 && B->dtype == MX_E2M1 && o.a_scale_layout == MX_SCALE_2D &&
+    else if (M <= kDecodeAutoM && A->dtype != MX_E2M1 && B->dtype == MX_E2M1 && o.a_scale_layout == MX_SCALE_2D &&
              o.b_scale_layout == MX_SCALE_2D && Bs->stride[0] == 1 && As->stride[1] == 1 && K % 512 == 0 &&
              N % 16 == 0 && Bs->stride[1] % 16 == 0 && ((uintptr_t)Bs->ptr) % 16 == 0 &&
              N * b_ld < ((int64_t)1 << 31) && As->stride[0] % 16 == 0 && ((uintptr_t)As->ptr) % 16 == 0)
@@ -430,7 +437,8 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
   }
 
   if (kernel == MX_KERNEL_DECODE) {
-    if (M > 32) return set_error(MX_ERR_SHAPE, "the decode kernel handles M <= 32 (got %lld)", (long long)M);
+    if (M > kDecodeMaxM)
+      return set_error(MX_ERR_SHAPE, "the decode kernel handles M <= %lld (got %lld)", (long long)kDecodeMaxM, (long long)M);
     if (o.a_scale_layout != MX_SCALE_2D || o.b_scale_layout != MX_SCALE_2D || Bs->stride[0] != 1 ||
         As->stride[1] != 1)
       return set_error(MX_ERR_LAYOUT, "the decode kernel reads K-contiguous 2-D scales in place");
@@ -444,7 +452,19 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
     d.M = (int32_t)M; d.N = (int32_t)N; d.K = (int32_t)K;
     d.ldx = a_ld; d.ldxs = As->stride[0]; d.ldw = b_ld; d.ldws = Bs->stride[1]; d.ldc = C->stride[0];
     d.x_fmt = A->dtype; d.w_fmt = B->dtype; d.c_dtype = C->dtype; d.accumulate = o.accumulate;
-    if (K <= kDecodeChunk) return launch_gemm_decode(d, (hipStream_t)stream);
+    const int c_bytes = C->dtype == MX_BF16 ? 2 : 4;
+    // slabs of 32 rows of X (and of C, or of the chunk buffer)
+    auto launch_slabs = [&](const DecodeArgs& full, int out_bytes) {
+      for (int64_t m0 = 0; m0 < M; m0 += 32) {
+        DecodeArgs s = full;
+        s.X = full.X + m0 * full.ldx; s.Xs = full.Xs + m0 * full.ldxs;
+        s.C = (uint8_t*)full.C + m0 * full.ldc * out_bytes;
+        s.M = (int32_t)(M - m0 < 32 ? M - m0 : 32);
+        if (int rc = launch_gemm_decode(s, (hipStream_t)stream)) return rc;
+      }
+      return (int)MX_OK;
+    };
+    if (K <= kDecodeChunk) return launch_slabs(d, c_bytes);
     // a longer K (the down-projection of an MoE layer, K = 14336 / 28672): chunks of kDecodeChunk elements, each
     // streaming its part of the weights once, summed in fp32 in the workspace in chunk order
     const int64_t need = decode_partial_bytes(M, N, K, o);
@@ -458,7 +478,7 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
       c.W = d.W + k0 / 2; c.Ws = d.Ws + k0 / 32;      // FP4 weights: two elements per byte
       c.K = (int32_t)(K - k0 < kDecodeChunk ? K - k0 : kDecodeChunk);
       c.C = workspace; c.ldc = N; c.c_dtype = MX_F32; c.accumulate = k0 > 0;
-      if (int rc = launch_gemm_decode(c, (hipStream_t)stream)) return rc;
+      if (int rc = launch_slabs(c, 4)) return rc;
     }
     return launch_splitk_reduce((const float*)workspace, 1, M, N, C->ptr, C->stride[0], C->dtype, o.accumulate,
                                 (hipStream_t)stream);

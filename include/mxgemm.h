@@ -105,7 +105,10 @@ enum {
   MX_KERNEL_MFMA_128x128 = 2, /* v_mfma_scale tiles, 128x128 macro tile, 4 waves                */
   MX_KERNEL_MFMA_256x256 = 3, /* 256x256 macro tile, 8 waves                                    */
   MX_KERNEL_MFMA_256x256_W4 = 4, /* 256x256 macro tile, 4 waves                                 */
-  MX_KERNEL_DECODE = 5,       /* skinny-M (M <= 32) weight-streaming kernel                     */
+  MX_KERNEL_DECODE = 5,       /* skinny-M weight-streaming kernel: 8-bit activations x FP4 weights,
+                                 K % 512 == 0, N % 16 == 0; 32 rows of A and 8192 of K per launch, more
+                                 rows (up to 128; MX_KERNEL_AUTO: up to 64) in slabs, a longer K in chunks
+                                 summed in fp32 in the workspace                                  */
   MX_KERNEL_MFMA_PINGPONG = 6, /* 256x256 macro tile, two 4-wave teams alternating LDS/MFMA phases,
                                  v_mfma_scale_f32_16x16x128_f8f6f4                                */
   MX_KERNEL_MFMA_PINGPONG32 = 7, /* the same schedule on v_mfma_scale_f32_32x32x64_f8f6f4; 8-bit
@@ -144,7 +147,8 @@ MX_API int mx_device_check(void);
 
 /*
  * Bytes of device workspace mx_gemm needs for the given problem (native re-layout of the scale
- * tensors).  0 if both scale tensors are already in a native layout or the generic kernel is used.
+ * tensors, split-K partial products, the fp32 chunk sums of the skinny-M kernel for K > 8192).  0 if both
+ * scale tensors are already in a native layout and nothing else is needed, or the generic kernel is used.
  */
 MX_API int64_t mx_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, const mx_gemm_opts* opts);
 

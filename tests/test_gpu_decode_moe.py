@@ -52,6 +52,23 @@ def test_decode_long_k_accumulate_and_static_scratch(ct, dev):
     assert torch.equal(c, c2) and O.rel_fro(c.cpu(), ref) <= 1e-3
 
 
+@pytest.mark.parametrize("M,N,K,kernel", [(48, 528, 4096, "auto"), (64, 1040, 8192, "auto"), (33, 64, 14336, "auto"),
+                                          (100, 272, 2048, "decode"), (128, 64, 9216, "decode")])
+def test_decode_more_than_32_rows(ct, dev, M, N, K, kernel):
+    """More than 32 rows of X run slab by slab on the same kernel (the automatic choice up to 64 rows)."""
+    x = randn_operand(M, K, O.E4M3, 281, dev)
+    w = randn_operand(N, K, O.E2M1, 282, dev, std=0.02)
+    ref = oracle_matmul(x, w)
+    for out_dtype, tol in ((torch.float32, 1e-3), (torch.bfloat16, 8e-3)):
+        c = ct.block_scaled_matmul(x.storage, x.scale_t, w.storage.T, w.scale_t.T, b_format="e2m1",
+                                   out_dtype=out_dtype, kernel=kernel)
+        assert O.rel_fro(c.float().cpu(), ref) <= tol
+        # the slabs are what single calls on 32 rows give
+        c0 = ct.block_scaled_matmul(x.storage[:32], x.scale_t[:32], w.storage.T, w.scale_t.T, b_format="e2m1",
+                                    out_dtype=out_dtype, kernel="decode")
+        assert torch.equal(c[:32], c0)
+
+
 def test_decode_accumulate(ct, dev):
     x = randn_operand(32, 1024, O.E4M3, 83, dev)
     w = randn_operand(64, 1024, O.E2M1, 84, dev)

@@ -364,7 +364,7 @@ def test_drop_in_signature_caches_scale_relayout(ct, dev):
     c2 = ct.cutile_block_scaled_matmul(a.storage, a_sw, b.storage.T, b_sw)
     assert c1.dtype == torch.float32 and torch.equal(c1, want) and torch.equal(c2, want)
     assert len(ops._SCALE_CACHE._entries) == 2
-    torch.testing.assert_close(c1.cpu(), oracle_matmul(a, b), atol=1e-4, rtol=1e-3)
+    assert O.rel_fro(c1.cpu(), oracle_matmul(a, b)) <= 1e-3
     a_sw.view(torch.uint8).add_(1)                                              # every A scale doubled, through torch
     c3 = ct.cutile_block_scaled_matmul(a.storage, a_sw, b.storage.T, b_sw)
     assert torch.equal(c3, want * 2)
