@@ -375,6 +375,62 @@ def bench_shape(ct, O, dev, M, N, K, check, kernels=("auto", "mfma128", "pingpon
     return out
 
 
+def probe_mfma(ct, dev, reps=6):
+    """What the chip sustains on the scaled MFMA instruction out of registers alone (mx_probe_mfma_rate: the GEMM
+    kernel's register tile, two waves per SIMD, no LDS or memory traffic), for several kinds of operand bits.  The
+    chip lowers its clock as operand bits toggle, so the rate on real data is the ceiling of any GEMM schedule on that
+    data.  Each kind is run `reps` times back to back (about 20 ms each) and the last run is reported: by then the
+    power management has settled.  (The clock each kind ran at is in the rocprofv3 summary of this probe under
+    profiles/: SQ_BUSY_CYCLES over the launch's duration.)"""
+    import ctypes
+    lib = ct.lib()
+    n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
+    nbytes = 12 * 512 * 32
+    g = torch.Generator(device=dev).manual_seed(7)
+
+    def fp8_real():
+        q, _ = ct.block_quantize(torch.randn((192, 1024), generator=g, device=dev), 32, torch.float8_e4m3fn, scale_mode="floor")
+        return q.view(torch.uint8).reshape(-1)
+
+    def fp4_real():
+        q, _ = ct.block_quantize(torch.rand((96, 2048), generator=g, device=dev) * 12 - 6, 32, "e2m1", scale_mode="floor")
+        f = torch.zeros((12 * 512, 32), dtype=torch.uint8, device=dev)
+        f[:, :16] = q.reshape(12 * 512, 16)
+        return f.reshape(-1)
+
+    def fp4_random():
+        f = torch.zeros((12 * 512, 32), dtype=torch.uint8, device=dev)
+        f[:, :16] = torch.randint(0, 256, (12 * 512, 16), generator=g, device=dev, dtype=torch.uint8)
+        return f.reshape(-1)
+
+    kinds = [("mxfp8", "zeros", ct._lib.MX_E4M3, lambda: torch.zeros(nbytes, dtype=torch.uint8, device=dev)),
+             ("mxfp8", "uniform random bytes", ct._lib.MX_E4M3,
+              lambda: torch.randint(0, 256, (nbytes,), generator=g, device=dev, dtype=torch.uint8)),
+             ("mxfp8", "E4M3 of N(0,1), floor-rule block scales (the headline workload's data)", ct._lib.MX_E4M3, fp8_real),
+             ("mxfp4", "zeros", ct._lib.MX_E2M1, lambda: torch.zeros(nbytes, dtype=torch.uint8, device=dev)),
+             ("mxfp4", "uniform random nibbles", ct._lib.MX_E2M1, fp4_random),
+             ("mxfp4", "E2M1 of uniform(-6, 6), floor-rule block scales (the MXFP4 workload's data)", ct._lib.MX_E2M1, fp4_real)]
+    sink = torch.empty(n_cu * 512, dtype=torch.float32, device=dev)
+    out = []
+    for peak_key, name, fmt, make in kinds:
+        frags = make()
+        iters = 20000 if peak_key == "mxfp8" else 40000
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(reps):
+            e0.record()
+            rc = lib.mx_probe_mfma_rate(fmt, frags.data_ptr(), n_cu, iters, sink.data_ptr(),
+                                        torch.cuda.current_stream(dev).cuda_stream)
+            if rc != 0:
+                raise SystemExit("bench: " + ct._lib.last_error())
+            e1.record()
+            _sync()
+        ms = e0.elapsed_time(e1)
+        flop = n_cu * 8 * iters * 32 * 65536.0
+        tf = flop / ms * 1e-9
+        out.append({"format": peak_key, "data": name, "ms": ms, "tflops": tf, "frac_of_nominal_peak": tf / PEAK_TFLOPS[peak_key]})
+    return out
+
+
 def bench_decode(ct, O, dev, steps, warmup, check, M=32, N=28672, K=8192, nsets=8):
     """Decode-shaped mixed GEMM: X MXFP8 (M, K) x W MXFP4 (N, K)^T, bf16 out; the headline shape is 32 x 28672 x 8192.
     HBM bound; its 121 MiB working set fits in the Infinity Cache, so several weight sets are rotated.  Shapes the
@@ -545,6 +601,9 @@ def main():
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (a known-size reference for "
                          "scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    ap.add_argument("--probe-mfma", action="store_true",
+                    help="only run the register-only MFMA rate probe (what the chip sustains on zeros / random / real "
+                         "operand bits with nothing but the matrix pipe working) and print its JSON line")
     a = ap.parse_args()
     SETTLE_S = a.settle_ms * 1e-3
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -558,6 +617,10 @@ def main():
     torch.cuda.set_device(dev)
     if ct.lib().mx_device_check() != 0:
         raise SystemExit("bench.py: " + ct._lib.last_error())
+    if a.probe_mfma:
+        print(json.dumps({"probe": "mx_probe_mfma_rate: v_mfma_scale_f32_16x16x128_f8f6f4 out of registers, 8 waves per CU",
+                          "results": probe_mfma(ct, dev)}))
+        return
     if a.calib_copy:
         src = torch.empty(64 << 20, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)

@@ -19,7 +19,7 @@ CSRC = ROOT / "csrc"
 INCLUDE = ROOT.parent / "include"
 OUT = ROOT / "cutile_amd" / "libmxgemm.so"
 OBJ = ROOT / "build"
-SOURCES = ["mx_api.hip", "mx_gemm_mfma.hip", "mx_gemm_pp.hip", "mx_gemm_pp32.hip", "mx_gemm_w4.hip", "mx_gemm_generic.hip", "mx_gemm_decode.hip", "mx_aux.hip"]
+SOURCES = ["mx_api.hip", "mx_gemm_mfma.hip", "mx_gemm_pp.hip", "mx_gemm_pp32.hip", "mx_gemm_w4.hip", "mx_gemm_generic.hip", "mx_gemm_decode.hip", "mx_aux.hip", "mx_probe.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          f"-I{INCLUDE}", f"-I{CSRC}", "-Wno-unused-command-line-argument"]

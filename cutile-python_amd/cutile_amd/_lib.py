@@ -80,6 +80,8 @@ SYMBOLS = {
                                     ctypes.c_int64, ctypes.c_void_p]),
     "mx_quantize": (ctypes.c_int, [_P(MxTensor)] * 3 + [ctypes.c_int32, ctypes.c_void_p]),
     "mx_silu_mul_quantize": (ctypes.c_int, [_P(MxTensor)] * 3 + [ctypes.c_int32, ctypes.c_void_p]),
+    "mx_probe_mfma_rate": (ctypes.c_int, [ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32,
+                                          ctypes.c_void_p, ctypes.c_void_p]),
     "mx_packed_scale_bytes": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int64]),
     "mx_pack_scales": (ctypes.c_int, [_P(MxTensor), ctypes.c_int32, ctypes.c_int64, ctypes.c_int64,
                                       ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p]),

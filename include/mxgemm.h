@@ -307,6 +307,20 @@ MX_API int64_t mx_packed_scale_bytes(int64_t rows, int64_t K);
 MX_API int mx_pack_scales(const mx_tensor* scale, int32_t layout, int64_t rows, int64_t K, int32_t native_layout,
                    int32_t operand, void* packed, void* stream);
 
+/*
+ * Measurement aid (no reference counterpart; the reference measures whole kernels only, cext/tile_kernel.cpp:3921-4042):
+ * the rate at which the chip runs v_mfma_scale_f32_16x16x128_f8f6f4 out of registers alone on the given operand bits
+ * -- no LDS, no memory traffic -- i.e. the ceiling that the data itself (through the chip's power management) puts
+ * on any GEMM schedule.  `workgroups` workgroups of 8 waves (two per SIMD, one workgroup per CU when workgroups =
+ * the CU count) each load 8 + 4 operand fragments per wave from `frags` (12 x 512 fragments of 32 bytes, [fragment]
+ * [thread]; MX_E2M1 uses the first 16 bytes of each; unit scales) and multiply all 32 pairs `iters` times:
+ * workgroups x 8 x iters x 32 x 65536 flop per launch.  sink[workgroups x 512] receives a value that keeps the
+ * products alive.  Asynchronous on `stream`; time it with events, and take the clock it ran at from the
+ * SQ_BUSY_CYCLES counter of a profiler run over the launch's duration.
+ */
+MX_API int mx_probe_mfma_rate(int32_t fmt, const void* frags, int32_t workgroups, int32_t iters, float* sink,
+                       void* stream);
+
 #ifdef __cplusplus
 }
 #endif
