@@ -379,7 +379,8 @@ int gemm_impl(const mx_tensor* A, const mx_tensor* As, const mx_tensor* B, const
   int kernel = o.kernel;
   if (kernel == MX_KERNEL_AUTO) {
     if (why) kernel = MX_KERNEL_GENERIC;
-    else if (M <= kDecodeAutoM && A->dtype != MX_E2M1 && B->dtype == MX_E2M1 && o.a_scale_layout == MX_SCALE_2D &&
+    else if (M <= kDecodeAutoM && o.split_k <= 1 && A->dtype != MX_E2M1 && B->dtype == MX_E2M1 &&
+             o.a_scale_layout == MX_SCALE_2D &&
              o.b_scale_layout == MX_SCALE_2D && Bs->stride[0] == 1 && As->stride[1] == 1 && K % 512 == 0 &&
              N % 16 == 0 && Bs->stride[1] % 16 == 0 && ((uintptr_t)Bs->ptr) % 16 == 0 &&
              N * b_ld < ((int64_t)1 << 31) && As->stride[0] % 16 == 0 && ((uintptr_t)As->ptr) % 16 == 0)
