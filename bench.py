@@ -434,14 +434,14 @@ def probe_mfma(ct, dev, reps=6):
 def bench_decode(ct, O, dev, steps, warmup, check, M=32, N=28672, K=8192, nsets=8):
     """Decode-shaped mixed GEMM: X MXFP8 (M, K) x W MXFP4 (N, K)^T, bf16 out; the headline shape is 32 x 28672 x 8192.
     HBM bound; its 121 MiB working set fits in the Infinity Cache, so several weight sets are rotated.  Shapes the
-    skinny-M kernel does not take (M > 32) run on what MX_KERNEL_AUTO picks, with the weight scales packed once."""
+    skinny-M kernel is not chosen for (M > 64) run on what MX_KERNEL_AUTO picks, with the weight scales packed once."""
     x_q, x_s = _quantized(ct, M, K, torch.float8_e4m3fn, 2001, dev, "randn")
     nsets = max(nsets, -(-(300 << 20) // (N * K // 2)))
     ws = []
     for i in range(nsets):
         w_q, w_s = _quantized(ct, N, K, "e2m1", 2002 + i, dev, "randn", std=0.02, cpu_seeded=(i == 0))
         ws.append((w_q, w_s, torch.empty((M, N), dtype=torch.bfloat16, device=dev),
-                   w_s.T if M <= 32 else ct.pack_scales(w_s, operand="b")))
+                   w_s.T if M <= 64 else ct.pack_scales(w_s, operand="b")))
     err = None
     if check:
         w_q, w_s, c, w_sc = ws[0]
