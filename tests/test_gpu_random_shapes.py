@@ -62,3 +62,49 @@ def test_random_problems_match_oracle(ct, dev, seed):
         ran += 1
     print(f"seed {seed}: {ran} problems checked, {refused} refused", flush=True)
     assert ran >= 10
+
+
+@pytest.mark.parametrize("seed", [21, 22, 23])
+def test_random_moe_routings_match_oracle(ct, dev, seed):
+    """Grouped GEMM on random routings: token count, expert count, top-k, tile_m, kernel, weight format, skew of the
+    router (experts that get nothing, one expert that gets most), trimmed or worst-case-length slot arrays, routed
+    weights.  Every routed row must be written (C starts as NaN) and is compared with the oracle."""
+    rnd = random.Random(seed)
+    for case in range(10):
+        E = rnd.choice([1, 2, 5, 8, 16, 64])
+        topk = rnd.choice([k for k in (1, 2, 4, 8) if k <= E])
+        T = rnd.choice([1, 3, 17, 48, 130, 300])
+        K = rnd.choice([128, 512, 1024])
+        N = rnd.choice([64, 256, 320, 1024])
+        wf = rnd.choice([O.E4M3, O.E4M3, O.E2M1])
+        kernel, tile = rnd.choice([("generic", 16), ("mfma128", 128), ("mfma128", 256), ("mfma256", 256),
+                                   ("mfma256w4", 256), ("pingpong", 256), ("auto", 128), ("auto", 256)])
+        out = rnd.choice([torch.float32, torch.bfloat16])
+        exact, routed = rnd.random() < 0.5, rnd.random() < 0.5
+        skew = rnd.choice([0.0, 0.0, 2.0, 8.0])
+        what = (f"seed {seed} case {case}: T={T} E={E} top{topk} K={K} N={N} w={wf} {kernel} tile_m={tile} {out} "
+                f"exact={exact} routed_weights={routed} skew={skew}")
+        print(what, flush=True)
+        a = randn_operand(T, K, O.E4M3, 1000 * seed + 3 * case, dev, std=0.5)
+        w = randn_operand(E * N, K, wf, 1000 * seed + 3 * case + 1, dev, std=0.1)
+        g = torch.Generator().manual_seed(1000 * seed + 3 * case + 2)
+        logits = torch.rand((T, E), generator=g)
+        logits[:, 0] += skew                      # expert 0 takes (nearly) every token ...
+        if E > 2:
+            logits[:, E - 1] -= 10.0              # ... and the last expert none
+        ids = torch.topk(logits, topk, dim=1).indices
+        tw = torch.rand((T, topk), generator=g) if routed else None
+        ref = O.grouped_reference(a.codes, a.scales, w.codes.reshape(E, N, K), w.scales.reshape(E, N, K // 32),
+                                  ids.numpy(), w_fmt=wf)
+        if routed:
+            ref = ref * tw.reshape(-1, 1)
+        W = w.storage.view(E, N, -1)
+        Ws = w.scale_t.view(E, N, K // 32)
+        sid, eid = ct.moe_align_tile_size(ids.to(dev), tile, E, exact=exact)
+        C = torch.full((T, topk, N), float("nan"), device=dev, dtype=out)
+        ct.invoke_fused_moe_scaled(a.storage, a.scale_t, W, Ws, C, None if tw is None else tw.to(dev), sid, eid, routed,
+                                   topk, tile, kernel=kernel, b_format="e2m1" if wf == O.E2M1 else None)
+        got = C.view(-1, N).float().cpu()
+        assert not torch.isnan(got).any(), f"{what}: a routed row was not written"
+        err = O.rel_fro(got, ref)
+        assert err <= TOL[out], f"{what}: relative Frobenius error {err:.3e}"
